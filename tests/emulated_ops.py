@@ -185,3 +185,162 @@ def sample(logits, temperature, keys, out):
             if v > best:
                 best, besti = v, i
         out[row] = besti
+
+
+# ---------------------------------------------------------------- norm after the sum, recurrence, latent attention, experts
+
+def scaled_add_rmsnorm(residual, pending, alpha, weight, eps, out):
+    r = alpha * residual
+    if pending is not None:
+        r = r + (pending.sum(0) if pending.dim() == 3 else pending.float())
+    y = r / torch.sqrt(r.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    residual.copy_(y)
+    if out is not None:
+        out.copy_(y.to(out.dtype))
+
+
+def mlstm_scan(qkv, k_off, v_off, gates, state, slots, req_indptr, out, heads, dim, vdim, cap, qscale, denom_eps):
+    squash = (lambda z: cap * torch.tanh(z / cap)) if cap else (lambda z: z)
+    for r in range(req_indptr.numel() - 1):
+        st = state[int(slots[r])]
+        S = st[:, : dim * vdim].reshape(heads, dim, vdim).clone()
+        n = st[:, dim * vdim: dim * vdim + dim].clone()
+        m = st[:, dim * vdim + dim].clone()
+        for t in range(int(req_indptr[r]), int(req_indptr[r + 1])):
+            q = qkv[t, : heads * dim].float().view(heads, dim) * qscale
+            k = qkv[t, k_off: k_off + heads * dim].float().view(heads, dim)
+            v = qkv[t, v_off: v_off + heads * vdim].float().view(heads, vdim)
+            i = squash(gates[t, :heads])
+            f = torch.nn.functional.logsigmoid(squash(gates[t, heads:]))
+            m_new = torch.maximum(f + m, i)
+            keep, take = torch.exp(f + m - m_new), torch.exp(i - m_new)
+            S = keep[:, None, None] * S + take[:, None, None] * k[:, :, None] * v[:, None, :]
+            n = keep[:, None] * n + take[:, None] * k
+            m = m_new
+            den = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + denom_eps
+            out[t] = (torch.einsum("hdv,hd->hv", S, q) / den[:, None]).reshape(-1)
+        st[:, : dim * vdim] = S.reshape(heads, -1)
+        st[:, dim * vdim: dim * vdim + dim] = n
+        st[:, dim * vdim + dim] = m
+
+
+def gated_head_norm(o, gate, weight, eps, out, heads, vdim):
+    T = o.shape[0]
+    x = o.view(T, heads, vdim)
+    y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_((y.reshape(T, -1) * weight.float() * torch.sigmoid(gate.float())).to(out.dtype))
+
+
+LATENT_ATTENTION_ROWS = 16
+LATENT_MAX_RANK = 1024
+ACTIVATIONS = {"none": 0, "relu2": 1}
+
+
+def latent_tile_tokens(heads):
+    return max(1, LATENT_ATTENTION_ROWS // min(heads, LATENT_ATTENTION_ROWS))
+
+
+def _turn(x, positions, inv_freq):
+    """x [T, ..., rot]: the first 2 * len(inv_freq) entries turned in neighbouring pairs."""
+    d = 2 * inv_freq.numel()
+    ang = positions.float()[:, None] * inv_freq[None, :]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [d // 2]
+    c, s = ang.cos().view(shape), ang.sin().view(shape)
+    u, v = x[..., 0:d:2], x[..., 1:d:2]
+    y = x.clone()
+    y[..., 0:d:2] = u * c - v * s
+    y[..., 1:d:2] = v * c + u * s
+    return y
+
+
+def latent_prepare(down, q_rank, rank, rot, rot_dims, wq, wkv, eps, positions, inv_freq, cq, token_req=None, block_table=None,
+                   plane=None, page_size=0):
+    x = down.float()
+    norm = lambda t, w: t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    cq.copy_(norm(x[:, :q_rank], wq).to(cq.dtype))
+    if plane is None:
+        return
+    c = norm(x[:, q_rank: q_rank + rank], wkv)
+    kr = _turn(x[:, q_rank + rank: q_rank + rank + rot], positions, inv_freq)
+    row = torch.cat((c, kr), dim=-1).to(plane.dtype)
+    for t in range(down.shape[0]):
+        p = int(positions[t])
+        page = int(block_table[int(token_req[t]), p // page_size])
+        if page:
+            plane[page, 0, p % page_size] = row[t]
+
+
+def rotate_pairs(src, src_head, src_off, dst, dst_head, dst_off, positions, inv_freq, heads, rot):
+    T = src.shape[0]
+    x = torch.stack([src[:, h * src_head + src_off: h * src_head + src_off + rot] for h in range(heads)], dim=1).float()
+    y = _turn(x, positions, inv_freq).to(dst.dtype)
+    for h in range(heads):
+        dst[:, h * dst_head + dst_off: h * dst_head + dst_off + rot] = y[:, h]
+
+
+def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles, tile_tokens, heads, rank, rot,
+                     page_size, scale, sink, splits=1):
+    D = rank + rot
+    for tile in range(num_tiles):
+        if tile_req is None:
+            r, t0, first, n_new = tile, 0, tile, 1
+        else:
+            r = int(tile_req[tile]); t0 = int(tile_tok0[tile])
+            first = int(req_indptr[r]); n_new = int(req_indptr[r + 1]) - first
+        ctx = int(ctx_lens[r])
+        for i in range(t0, min(t0 + tile_tokens, n_new)):
+            pos = ctx + i
+            keys = torch.arange(0, pos + 1)
+            rows = plane[block_table[r, keys // page_size].long(), 0, keys % page_size].float()     # [n, D]
+            s = (q[first + i].float().view(heads, D) @ rows.T) * scale
+            top = s.max(-1, keepdim=True).values
+            if sink is not None:
+                top = torch.maximum(top, sink[:, None])
+            e = torch.exp(s - top)
+            den = e.sum(-1, keepdim=True) + (torch.exp(sink[:, None] - top) if sink is not None else 0.0)
+            out[first + i] = ((e / den) @ rows[:, :rank]).reshape(-1).to(out.dtype)
+
+
+def heads_linear(x, x_head, weight, out, out_head):
+    G, N, K = weight.shape
+    for g in range(G):
+        out[:, g * out_head: g * out_head + N] = (x[:, g * x_head: g * x_head + K].float() @ weight[g].float().T).to(out.dtype)
+
+
+def _act(y, activation):
+    return torch.clamp(y, min=0) ** 2 if activation == "relu2" else y
+
+
+def experts_linear(x, slot_token, weight, offsets, out, activation="none"):
+    for e in range(weight.shape[0]):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            rows = x[slot_token[lo:hi].long()] if slot_token is not None else x[lo:hi]
+            out[lo:hi] = _act(rows.float() @ weight[e].float().T, activation).to(out.dtype)
+
+
+def route(logits, top):
+    T, E = logits.shape
+    best = logits.topk(top, dim=-1)               # ties: not met in tests
+    weights = torch.softmax(best.values, dim=-1)
+    chosen = best.indices.reshape(-1)
+    order = torch.sort(chosen, stable=True).indices
+    slot_token = (order // top).to(torch.int32)
+    pair_slot = torch.empty(T * top, dtype=torch.int32)
+    pair_slot[order] = torch.arange(T * top, dtype=torch.int32)
+    offsets = torch.zeros(E + 1, dtype=torch.int32)
+    offsets[1:] = torch.bincount(chosen, minlength=E).cumsum(0)
+    return weights, offsets, slot_token, pair_slot
+
+
+def combine(y, pair_slot, weights, out):
+    T, top = weights.shape
+    out.copy_((y[pair_slot.long()].float().view(T, top, -1) * weights[:, :, None]).sum(1).to(out.dtype))
+
+
+def activation(x, kind):
+    x.copy_(_act(x.float(), kind).to(x.dtype))
+
+
+def compute_units():
+    return 256

@@ -29,9 +29,11 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class RMSNormSpec(PartSpec):
+    """``weight_name``: the norm's one tensor below the norm's own name; empty: the tensor bears the norm's name itself."""
     kind: ClassVar[str] = "rmsnorm"
     dim: int = 0
     eps: float = 1e-6
+    weight_name: str = "weight"
 
 
 @dataclass(frozen=True)
@@ -65,6 +67,74 @@ class SwiGLUSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class PairRotarySpec(PartSpec):
+    """Rotary position encoding in the interleaved layout: of the first ``dims`` entries of a vector, entry ``2i`` is
+    paired with ``2i + 1`` and turned by ``position * base**(-2i / dims)``; what lies beyond ``dims`` passes unchanged."""
+    kind: ClassVar[str] = "rope_pairs"
+    dims: int = 0
+    base: float = 10000.0
+
+
+@dataclass(frozen=True)
+class MLSTMSpec(PartSpec):
+    """Matrix-memory recurrence (the mLSTM of xLSTM): per head a ``dim x vdim`` state with exponential input gate, sigmoid
+    forget gate and a running maximum that starts at ``m_start``; gate pre-activations are capped by ``gate_cap * tanh(./gate_cap)``
+    (``None``: no cap); the output's denominator is ``max(|n.q|, exp(-m)) + denom_eps``; each head's output is divided by
+    its root mean square (``norm_eps``), multiplied by a weight and by a sigmoid gate."""
+    kind: ClassVar[str] = "mlstm"
+    hidden: int = 0
+    heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    gate_cap: float | None = None
+    norm_eps: float = 1e-6
+    denom_eps: float = 1e-6
+    query_scale: float | None = None     # None: dim ** -0.5
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec(PartSpec):
+    """Attention whose keys and values are up-projections of one cached latent per token (``kv_rank`` numbers, normed) beside one
+    rotated key part (``rot_dim`` numbers) that all heads share; queries come through a latent of ``q_rank`` numbers.  ``sink``:
+    the softmax's denominator also holds ``exp`` of one learned number per head."""
+    kind: ClassVar[str] = "latent_attention"
+    hidden: int = 0
+    heads: int = 0
+    dim: int = 0            # unrotated query/key dimensions per head
+    rot_dim: int = 0        # rotated ones
+    vdim: int = 0
+    kv_rank: int = 0
+    q_rank: int = 0
+    scale: float = 1.0
+    norm_eps: float = 1e-6
+    sink: bool = True
+    position: PartSpec | None = None     # encoding of the rotated parts
+
+
+@dataclass(frozen=True)
+class DenseFFSpec(PartSpec):
+    """``down(act(up(h)))`` with an elementwise activation (``relu2``: the square of relu) and optional biases."""
+    kind: ClassVar[str] = "dense_ff"
+    hidden: int = 0
+    intermediate: int = 0
+    activation: str = "relu2"
+    bias: bool = True
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec(PartSpec):
+    """``experts`` small feed-forward layers ``down(act(up(h)))`` without biases; a linear router (with bias, in 32-bit)
+    picks the ``top`` largest logits per token, whose softmax (over the chosen ones only) weighs the experts' outputs."""
+    kind: ClassVar[str] = "routed_experts"
+    hidden: int = 0
+    intermediate: int = 0
+    experts: int = 0
+    top: int = 1
+    activation: str = "relu2"
+    router_bias: bool = True
+
+
+@dataclass(frozen=True)
 class BlockSpec(PartSpec):
     """One layer: a mixer and a feed-forward, each behind its own norm.
 
@@ -79,6 +149,14 @@ class BlockSpec(PartSpec):
     ffn_name: str = "mlp"
     mixer_norm_name: str = "input_layernorm"
     ffn_norm_name: str = "post_attention_layernorm"
+
+
+@dataclass(frozen=True)
+class PostNormBlockSpec(BlockSpec):
+    """One layer with the norm after the sum: ``x <- norm1(alpha * x + mixer(x))``, then ``x <- norm2(alpha * x + ffn(x))``;
+    the sublayers read ``x`` itself.  ``ffn`` (and then ``ffn_norm``) may be ``None``: the layer ends after the first step."""
+    kind: ClassVar[str] = "postnorm_residual"
+    alpha: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -110,6 +188,11 @@ class ModelSpec:
     embed_scale: float = 1.0       # factor on the embedding rows as they enter the residual stream
     logit_scale: float = 1.0       # factor on the logits (applied to the final norm's output, in 32-bit)
     head_bias: bool = False        # the output head has a bias vector ``<head_name>.bias``
+    weight_suffix: str = "weight"  # the embedding's and the head's matrix below their names; empty: the tensor bears the name itself
+    layers_format: str = ""        # the name of layer i as a format string (``"l{}"``); empty: ``<layers_prefix>.<i>``
+
+    def layer_name(self, i: int) -> str:
+        return self.layers_format.format(i) if self.layers_format else f"{self.layers_prefix}.{i}"
 
     def __post_init__(self):
         for i, e in enumerate(self.order):

@@ -512,3 +512,53 @@ extern "C" int tl_stream_read(const void* data, size_t bytes, void* sink, int gr
     TL_CHECK_LAUNCH("stream_read");
     return TL_OK;
 }
+
+// ------------------------------------------------------------------ norm after the sum
+// x <- norm(alpha * x + y) * weight, row by row: the layer arrangement in which the norm follows the sum and the
+// sublayers read the normed stream itself.  `residual` (float) holds x and receives the result; `out` (optional)
+// receives its rounding to the activation type, which the next sublayer's products read.  y comes as one tensor of
+// the activation type (parts == 0), as float slabs of partial sums, or not at all.
+template <typename T>
+__global__ void scaled_add_rmsnorm_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
+                                          float alpha, const void* __restrict__ weight, int weight_f32, float eps,
+                                          T* __restrict__ out, int hidden) {
+    __shared__ float red[16];
+    const int row = blockIdx.x;
+    float* res = residual + (size_t)row * hidden;
+    const T* pen = (pending && parts == 0) ? (const T*)pending + (size_t)row * hidden : nullptr;
+    const float* pparts = (pending && parts > 0) ? (const float*)pending + (size_t)row * hidden : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float r = alpha * res[i];
+        if (pen) r += to_float(pen[i]);
+        if (pparts) {
+            float y = 0.f;
+            for (int p = 0; p < parts; ++p) y += pparts[p * part_stride + i];
+            r += y;
+        }
+        res[i] = r;                      // the same thread reads it back below
+        ss = fmaf(r, r, ss);
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float y = res[i] * inv * load_vec(weight, weight_f32, i);
+        res[i] = y;
+        if (out) out[(size_t)row * hidden + i] = from_float<T>(y);
+    }
+}
+
+extern "C" int tl_scaled_add_rmsnorm(void* residual, const void* pending, int parts, int total_rows, float alpha, const void* weight,
+                                     int weight_f32, float eps, void* out, int rows, int hidden, int dtype, hipStream_t stream) {
+    TL_REQUIRE(rows >= 0 && hidden > 0 && parts >= 0, "scaled_add_rmsnorm: bad sizes rows=%d hidden=%d", rows, hidden);
+    if (rows == 0) return TL_OK;
+    const size_t part_stride = (size_t)total_rows * hidden;
+    dim3 grid(rows), block(hidden <= 512 ? 128 : hidden <= 2048 ? 256 : 512);
+    if (dtype == TL_DT_F32)
+        scaled_add_rmsnorm_kernel<float><<<grid, block, 0, stream>>>((float*)residual, pending, parts, part_stride, alpha, weight, weight_f32, eps, (float*)out, hidden);
+    else if (dtype == TL_DT_BF16)
+        scaled_add_rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((float*)residual, pending, parts, part_stride, alpha, weight, weight_f32, eps, (bf16_t*)out, hidden);
+    else TL_REQUIRE(false, "scaled_add_rmsnorm: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("scaled_add_rmsnorm");
+    return TL_OK;
+}

@@ -1,0 +1,219 @@
+// Matrix products over groups (one weight matrix per group: an expert and the tokens routed to it, or a head and
+// its slice of every token's row), the router's choice of experts, the sort of tokens by expert, the weighted sum
+// of the chosen experts' outputs, and the elementwise activation of a dense feed-forward.  Sums are float.
+#include "common.h"
+
+#define ACT_NONE 0
+#define ACT_RELU2 1
+
+__device__ __forceinline__ float activate(float v, int act) {
+    if (act == ACT_RELU2) { v = fmaxf(v, 0.f); return v * v; }
+    return v;
+}
+
+// ------------------------------------------------------------------ grouped product
+// out[row(m), g_out + n] = act(sum_k a[src(m), g_a + k] * w[g][n][k]) for the rows m of group g, in tiles of 64 x 64
+// with K in steps of 16 through shared memory; a thread owns a 4 x 4 block of the tile.  One order of summation per
+// output element whatever else is in the step.
+//   offsets == null: every group has the same `rows` rows (row m is token m), group g reads the columns from
+//                    g * a_group on and writes the columns from g * out_group on; blockIdx.z is the group.
+//   offsets != null: group g owns the rows offsets[g] .. offsets[g + 1] - 1 (sorted slots); blockIdx.x runs over an upper
+//                    bound of all groups' tiles and finds its group by walking the offsets; `src` (optional) maps a
+//                    sorted slot to the row of `a` it reads (a token routed to an expert), output rows are the slots.
+#define GG_T 64
+#define GG_K 16
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+grouped_gemm_kernel(const T* __restrict__ a, int a_ld, int a_group, const int* __restrict__ src, const T* __restrict__ w,
+                    T* __restrict__ out, int out_ld, int out_group, const int* __restrict__ offsets, int groups, int rows,
+                    int N, int K, int act) {
+    __shared__ float sa[GG_K][GG_T + 4];
+    __shared__ float sw[GG_K][GG_T + 4];
+    int g, m0, m_end;
+    if (offsets == nullptr) {
+        g = blockIdx.z; m0 = blockIdx.x * GG_T; m_end = rows;
+        if (m0 >= m_end) return;
+    } else {
+        int tile = blockIdx.x;
+        g = 0; m0 = -1; m_end = 0;
+        for (int e = 0; e < groups; ++e) {
+            const int lo = offsets[e], hi = offsets[e + 1], tiles = (hi - lo + GG_T - 1) / GG_T;
+            if (tile < tiles) { g = e; m0 = lo + tile * GG_T; m_end = hi; break; }
+            tile -= tiles;
+        }
+        if (m0 < 0) return;
+    }
+    const int n0 = blockIdx.y * GG_T;
+    const T* wg = w + (size_t)g * N * K;
+    const int a_col = offsets == nullptr ? g * a_group : 0, out_col = offsets == nullptr ? g * out_group : 0;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;      // the thread's block: rows ty*4.., columns tx*4..
+    // loads: a thread fetches 4 elements of a and 4 of w per step: row lr of the tile, k = lk .. lk+3
+    const int lr = threadIdx.x / 4, lk = (threadIdx.x % 4) * 4;
+    const int am = m0 + lr;
+    const T* arow = nullptr;
+    if (am < m_end) arow = a + (size_t)(src ? src[am] : am) * a_ld + a_col;
+    const T* wrow = (n0 + lr < N) ? wg + (size_t)(n0 + lr) * K : nullptr;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += GG_K) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = k0 + lk + u;
+            sa[lk + u][lr] = (arow && k < K) ? to_float(arow[k]) : 0.f;
+            sw[lk + u][lr] = (wrow && k < K) ? to_float(wrow[k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < GG_K; ++k) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { av[u] = sa[k][ty * 4 + u]; wv[u] = sw[k][tx * 4 + u]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= m_end) continue;
+        T* orow = out + (size_t)m * out_ld + out_col;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) orow[n] = from_float<T>(activate(acc[i][j], act));
+        }
+    }
+}
+
+extern "C" int tl_grouped_gemm(const void* a, int a_ld, int a_group, const void* src, const void* w, void* out, int out_ld, int out_group,
+                               const void* offsets, int groups, int rows, int N, int K, int act, int dtype, hipStream_t stream) {
+    TL_REQUIRE(groups > 0 && rows >= 0 && N > 0 && K > 0 && a_ld > 0 && out_ld > 0, "grouped_gemm: bad sizes");
+    TL_REQUIRE(act == ACT_NONE || act == ACT_RELU2, "grouped_gemm: unknown activation %d", act);
+    if (rows == 0) return TL_OK;
+    // with offsets, `rows` is the number of sorted slots in all groups together: every group may end in a partial tile
+    dim3 grid(offsets ? (rows + GG_T - 1) / GG_T + groups : (rows + GG_T - 1) / GG_T, (N + GG_T - 1) / GG_T, offsets ? 1 : groups), block(256);
+    if (dtype == TL_DT_F32)
+        grouped_gemm_kernel<float><<<grid, block, 0, stream>>>((const float*)a, a_ld, a_group, (const int*)src, (const float*)w, (float*)out, out_ld,
+                                                               out_group, (const int*)offsets, groups, rows, N, K, act);
+    else if (dtype == TL_DT_BF16)
+        grouped_gemm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)a, a_ld, a_group, (const int*)src, (const bf16_t*)w, (bf16_t*)out, out_ld,
+                                                                out_group, (const int*)offsets, groups, rows, N, K, act);
+    else TL_REQUIRE(false, "grouped_gemm: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("grouped_gemm");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ the router's choice
+// Per token (one wave): the `top` largest of its `experts` logits, largest first (the lower index wins a tie), and
+// the softmax over those alone.
+__global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int* __restrict__ chosen,
+                                  float* __restrict__ weights, int tokens) {
+    const int t = blockIdx.x * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
+    if (t >= tokens) return;
+    const float* z = logits + (size_t)t * experts;
+    float first = 0.f, sum = 0.f, mine = 0.f;           // lane j keeps the j-th choice's term
+    unsigned long long taken = 0;                       // bit i: this lane's expert lane + 64 * i is chosen already
+    for (int j = 0; j < top; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane, i = 0; e < experts; e += TL_WAVE, ++i) {
+            const float v = z[e];
+            if (!((taken >> i) & 1ull) && (v > best || (v == best && e < at))) { best = v; at = e; }
+        }
+#pragma unroll
+        for (int o = TL_WAVE / 2; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, TL_WAVE);
+            const int oa = __shfl_xor(at, o, TL_WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        if (at % TL_WAVE == lane) taken |= 1ull << (at / TL_WAVE);
+        if (j == 0) first = best;
+        const float p = expf(best - first);
+        sum += p;
+        if (lane == j) { chosen[(size_t)t * top + j] = at; mine = p; }
+    }
+    if (lane < top) weights[(size_t)t * top + lane] = mine / sum;
+}
+
+// Sort of the (token, choice) pairs by expert, by one work-group: offsets[e] .. offsets[e + 1] - 1 are the slots of
+// expert e, slot_token[slot] the token a slot reads, pair_slot[token * top + j] where the pair's output row lies.
+__global__ void __launch_bounds__(1024)
+route_sort_kernel(const int* __restrict__ chosen, int pairs, int top, int experts, int* __restrict__ offsets,
+                  int* __restrict__ slot_token, int* __restrict__ pair_slot) {
+    extern __shared__ int cursor[];                     // [experts + 1]
+    for (int e = threadIdx.x; e <= experts; e += blockDim.x) cursor[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += blockDim.x) atomicAdd(&cursor[chosen[i] + 1], 1);
+    __syncthreads();
+    if (threadIdx.x == 0)
+        for (int e = 0; e < experts; ++e) cursor[e + 1] += cursor[e];
+    __syncthreads();
+    for (int e = threadIdx.x; e <= experts; e += blockDim.x) offsets[e] = cursor[e];
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+        const int slot = atomicAdd(&cursor[chosen[i]], 1);
+        slot_token[slot] = i / top;
+        pair_slot[i] = slot;
+    }
+}
+
+extern "C" int tl_route(const void* logits, int tokens, int experts, int top, void* chosen, void* weights, void* offsets,
+                        void* slot_token, void* pair_slot, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && top <= experts && top <= TL_WAVE && experts <= 64 * TL_WAVE, "route: bad sizes (experts %d, top %d)", experts, top);
+    TL_REQUIRE((experts + 1) * sizeof(int) <= 64 * 1024, "route: too many experts (%d)", experts);
+    if (tokens == 0) return TL_OK;
+    route_topk_kernel<<<(tokens + 3) / 4, 4 * TL_WAVE, 0, stream>>>((const float*)logits, experts, top, (int*)chosen, (float*)weights, tokens);
+    TL_CHECK_LAUNCH("route_topk");
+    route_sort_kernel<<<1, 1024, (experts + 1) * sizeof(int), stream>>>((const int*)chosen, tokens * top, top, experts, (int*)offsets,
+                                                                       (int*)slot_token, (int*)pair_slot);
+    TL_CHECK_LAUNCH("route_sort");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ weighted sum of the chosen experts' outputs
+// out[t, :] = sum_j weights[t, j] * y[pair_slot[t * top + j], :], summed in the order of the choices.
+template <typename T>
+__global__ void combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_slot, const float* __restrict__ weights,
+                               T* __restrict__ out, int top, int width) {
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float a = 0.f;
+        for (int j = 0; j < top; ++j)
+            a = fmaf(weights[(size_t)t * top + j], to_float(y[(size_t)pair_slot[(size_t)t * top + j] * width + i]), a);
+        out[(size_t)t * width + i] = from_float<T>(a);
+    }
+}
+
+extern "C" int tl_combine(const void* y, const void* pair_slot, const void* weights, void* out, int tokens, int top, int width,
+                          int dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && top > 0 && width > 0, "combine: bad sizes");
+    if (tokens == 0) return TL_OK;
+    if (dtype == TL_DT_F32)
+        combine_kernel<float><<<tokens, 256, 0, stream>>>((const float*)y, (const int*)pair_slot, (const float*)weights, (float*)out, top, width);
+    else if (dtype == TL_DT_BF16)
+        combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)y, (const int*)pair_slot, (const float*)weights, (bf16_t*)out, top, width);
+    else TL_REQUIRE(false, "combine: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("combine");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ elementwise activation, in place
+template <typename T>
+__global__ void activation_kernel(T* __restrict__ x, size_t n, int act) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        x[i] = from_float<T>(activate(to_float(x[i]), act));
+}
+
+extern "C" int tl_activation(void* x, long n, int act, int dtype, hipStream_t stream) {
+    TL_REQUIRE(n >= 0 && (act == ACT_NONE || act == ACT_RELU2), "activation: bad arguments");
+    if (n == 0 || act == ACT_NONE) return TL_OK;
+    const int blocks = (int)((n + 1023) / 1024 < 8192 ? (n + 1023) / 1024 : 8192);
+    if (dtype == TL_DT_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, (size_t)n, act);
+    else if (dtype == TL_DT_BF16) activation_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, (size_t)n, act);
+    else TL_REQUIRE(false, "activation: unknown dtype %d", dtype);
+    TL_CHECK_LAUNCH("activation");
+    return TL_OK;
+}

@@ -32,7 +32,7 @@ def parse_args(argv=None):
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (each rounded up to whole pages)")
     p.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
-    p.add_argument("--max-requests", type=int, default=8, help="most requests live at a time (default 8)")
+    p.add_argument("--max-requests", type=int, default=4, help="most requests live at a time: cache slots, each with its state (default 4)")
     p.add_argument("--graphs", action="store_true", help="replay decode-only steps as captured HIP graphs")
     return p.parse_args(argv)
 

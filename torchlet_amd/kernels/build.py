@@ -44,6 +44,9 @@ def _targets(head_dims) -> dict[str, tuple[str, list[str]]]:
         "elementwise": ("elementwise.hip", []),
         "gemm": ("gemm.hip", []),
         "sampling": ("sampling.hip", []),
+        "recurrent": ("recurrent.hip", []),
+        "latent": ("latent.hip", []),
+        "experts": ("experts.hip", []),
     }
     for hd in head_dims:
         t[f"attention_hd{hd}"] = ("attention.hip", [f"-DTL_HEAD_DIM={hd}"])

@@ -718,3 +718,245 @@ def stream_read(data: torch.Tensor, groups: int = 0) -> torch.Tensor:
     sink = torch.empty(groups or lib.tl_stream_read_groups(), dtype=torch.int32, device=data.device)
     _check(lib, lib.tl_stream_read(_ptr(data), ctypes.c_size_t(data.numel() * data.element_size()), _ptr(sink), c_int(groups), _stream()))
     return sink
+
+
+# ------------------------------------------------------------- the norm after the sum
+
+def scaled_add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, alpha: float, weight: torch.Tensor, eps: float,
+                       out: torch.Tensor | None) -> None:
+    """``residual <- rmsnorm(alpha * residual + pending) * weight`` in place (float32 ``[T, H]``); ``out`` (optional, of the
+    activation dtype) receives the rounded result.  ``pending``: ``[T, H]`` of ``out``'s dtype (float32 without ``out``),
+    float32 slabs ``[P, T, H]`` of partial sums, or ``None``."""
+    T, H = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("scaled_add_rmsnorm: the residual must be contiguous float32")
+    act = out.dtype if out is not None else torch.float32
+    if out is not None and (out.shape != (T, H) or not out.is_contiguous()):
+        raise KernelError(f"scaled_add_rmsnorm: out must be contiguous [{T}, {H}], got {tuple(out.shape)}")
+    parts = 0
+    if pending is not None:
+        if pending.dim() == 3:
+            parts = pending.shape[0]
+            if pending.dtype != torch.float32 or pending.shape[1:] != residual.shape or not pending.is_contiguous():
+                raise KernelError(f"scaled_add_rmsnorm: partial sums {pending.dtype} {tuple(pending.shape)} are not float32 [P, {T}, {H}]")
+        elif pending.shape != residual.shape or pending.dtype != act or not pending.is_contiguous():
+            raise KernelError(f"scaled_add_rmsnorm: pending {pending.dtype} {tuple(pending.shape)} does not match the residual")
+    wf = _vec(weight, H, "scaled_add_rmsnorm weight")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_scaled_add_rmsnorm(_ptr(residual), _ptr(pending), c_int(parts), c_int(T), c_float(alpha), _ptr(weight), c_int(wf),
+                                          c_float(eps), _ptr(out), c_int(T), c_int(H), c_int(_DT[act]), _stream()))
+
+
+# ------------------------------------------------------------- matrix-memory recurrence
+
+def mlstm_scan(qkv: torch.Tensor, k_off: int, v_off: int, gates: torch.Tensor, state: torch.Tensor, slots: torch.Tensor,
+               req_indptr: torch.Tensor, out: torch.Tensor, heads: int, dim: int, vdim: int, cap: float | None,
+               qscale: float, denom_eps: float) -> None:
+    """The matrix-memory recurrence over the step's tokens, request by request from the state its slot holds:
+    ``qkv [T, >=]`` holds per token the queries at column 0 (``heads * dim``), the keys at ``k_off`` and the values at
+    ``v_off`` (``heads * vdim``); ``gates`` float32 ``[T, 2 * heads]`` the raw input and forget gates (bias added);
+    ``state`` float32 ``[slots, heads, dim * vdim + dim + 1]`` (S, n, m per head) is updated in place; ``out`` float32
+    ``[T, heads * vdim]`` receives ``S^T q / (max(|n.q|, exp(-m)) + denom_eps)``."""
+    T = qkv.shape[0]
+    R = req_indptr.numel() - 1
+    if qkv.stride(1) != 1 or qkv.shape[1] < max(heads * dim, k_off + heads * dim, v_off + heads * vdim):
+        raise KernelError("mlstm_scan: the rows of qkv do not hold queries, keys and values at the given columns")
+    if gates.dtype != torch.float32 or gates.shape != (T, 2 * heads) or not gates.is_contiguous():
+        raise KernelError(f"mlstm_scan: gates must be contiguous float32 [{T}, {2 * heads}]")
+    if out.dtype != torch.float32 or out.shape != (T, heads * vdim) or not out.is_contiguous():
+        raise KernelError(f"mlstm_scan: out must be contiguous float32 [{T}, {heads * vdim}]")
+    if state.dtype != torch.float32 or state.dim() != 3 or state.shape[1:] != (heads, dim * vdim + dim + 1) or state.stride(2) != 1 \
+            or state.stride(1) != dim * vdim + dim + 1:
+        raise KernelError(f"mlstm_scan: state {tuple(state.shape)} is not float32 [slots, {heads}, {dim * vdim + dim + 1}]")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_mlstm_scan(_ptr(qkv), c_int(qkv.stride(0)), c_int(k_off), c_int(v_off), _ptr(gates), _ptr(state),
+                                  ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(req_indptr), _ptr(out), c_int(R), c_int(heads),
+                                  c_int(dim), c_int(vdim), c_float(cap if cap else 0.0), c_float(qscale), c_float(denom_eps),
+                                  c_int(_dt(qkv, "mlstm_scan")), _stream()))
+
+
+def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, heads: int, vdim: int) -> None:
+    """``out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight[h] * sigmoid(gate[t, h])`` per token and head:
+    ``o`` float32 ``[T, heads * vdim]``, ``gate`` a row-strided view ``[T, heads * vdim]`` of ``out``'s dtype."""
+    T = o.shape[0]
+    if o.dtype != torch.float32 or o.shape != (T, heads * vdim) or not o.is_contiguous():
+        raise KernelError("gated_head_norm: o must be contiguous float32 [T, heads * vdim]")
+    if out.shape != o.shape or not out.is_contiguous() or gate.dtype != out.dtype or gate.shape != o.shape or gate.stride(1) != 1:
+        raise KernelError("gated_head_norm: gate and out do not fit")
+    wf = _vec(weight, heads * vdim, "gated_head_norm weight")
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_gated_head_norm(_ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(wf), c_float(eps), _ptr(out),
+                                       c_int(T), c_int(heads), c_int(vdim), c_int(_dt(out, "gated_head_norm")), _stream()))
+
+
+# ------------------------------------------------------------- attention over a cached latent
+
+LATENT_ATTENTION_ROWS = 16       # rows (tokens x heads) a work-group of the latent attention owns
+LATENT_MAX_RANK = 1024
+
+
+def latent_tile_tokens(heads: int) -> int:
+    """New tokens of one request that share a tile of the latent attention."""
+    return max(1, LATENT_ATTENTION_ROWS // min(heads, LATENT_ATTENTION_ROWS))
+
+
+def latent_prepare(down: torch.Tensor, q_rank: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor, wkv: torch.Tensor, eps: float,
+                   positions: torch.Tensor, inv_freq: torch.Tensor, cq: torch.Tensor, token_req: torch.Tensor | None = None,
+                   block_table: torch.Tensor | None = None, plane: torch.Tensor | None = None, page_size: int = 0) -> None:
+    """From the fused down-projection ``down [T, q_rank + rank + rot]``: ``cq = rmsnorm(down[:, :q_rank]) * wq`` and, with a
+    plane ``[pages, 1, page, rank + rot]``, the token's cache row ``[rmsnorm(down[:, q_rank:q_rank + rank]) * wkv, the last
+    rot numbers with the first rot_dims of them turned in pairs by the token's position]``."""
+    T = down.shape[0]
+    if down.stride(1) != 1 or down.shape[1] < q_rank + rank + rot or cq.shape != (T, q_rank) or cq.dtype != down.dtype or not cq.is_contiguous():
+        raise KernelError("latent_prepare: shapes do not fit")
+    _i32(positions, "positions", T)
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2 or rot_dims % 2 or rot_dims > rot:
+        raise KernelError("latent_prepare: inv_freq must be float32 [rot_dims / 2]")
+    bt_stride = 0
+    if plane is not None:
+        _i32(token_req, "token_req", T)
+        _i32(block_table, "block_table")
+        bt_stride = block_table.stride(0)
+        if plane.dtype != down.dtype or plane.dim() != 4 or tuple(plane.shape[1:]) != (1, page_size, rank + rot) or not plane.is_contiguous():
+            raise KernelError(f"latent_prepare: plane {tuple(plane.shape)} {plane.dtype} is not [pages, 1, {page_size}, {rank + rot}] {down.dtype}")
+    lib = _lib("latent")
+    _check(lib, lib.tl_latent_prepare(_ptr(down), c_int(down.stride(0)), c_int(q_rank), c_int(rank), c_int(rot), c_int(rot_dims),
+                                      _ptr(wq), c_int(_vec(wq, q_rank, "query latent norm")), _ptr(wkv), c_int(_vec(wkv, rank, "latent norm")),
+                                      c_float(eps), _ptr(positions), _ptr(inv_freq), _ptr(token_req), _ptr(block_table), c_int(bt_stride),
+                                      _ptr(plane), c_int(page_size), _ptr(cq), c_int(T), c_int(_dt(down, "latent_prepare")), _stream()))
+
+
+def rotate_pairs(src: torch.Tensor, src_head: int, src_off: int, dst: torch.Tensor, dst_head: int, dst_off: int,
+                 positions: torch.Tensor, inv_freq: torch.Tensor, heads: int, rot: int) -> None:
+    """Per token and head, ``rot`` numbers from ``src[t, h * src_head + src_off:]`` to ``dst[t, h * dst_head + dst_off:]``, the first
+    ``2 * len(inv_freq)`` of them turned in neighbouring pairs by ``position * inv_freq``."""
+    T = src.shape[0]
+    rot_dims = 2 * inv_freq.numel()
+    if src.dtype != dst.dtype or src.stride(1) != 1 or dst.stride(1) != 1 or dst.shape[0] != T or rot_dims > rot \
+            or src.shape[1] < (heads - 1) * src_head + src_off + rot or dst.shape[1] < (heads - 1) * dst_head + dst_off + rot:
+        raise KernelError("rotate_pairs: shapes do not fit")
+    _i32(positions, "positions", T)
+    if inv_freq.dtype != torch.float32:
+        raise KernelError("rotate_pairs: inv_freq must be float32")
+    lib = _lib("latent")
+    _check(lib, lib.tl_rotate_pairs(_ptr(src), c_int(src.stride(0)), c_int(src_head), c_int(src_off), _ptr(dst), c_int(dst.stride(0)),
+                                    c_int(dst_head), c_int(dst_off), _ptr(positions), _ptr(inv_freq), c_int(T), c_int(heads), c_int(rot),
+                                    c_int(rot_dims), c_int(_dt(src, "rotate_pairs")), _stream()))
+
+
+def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, block_table: torch.Tensor, req_indptr: torch.Tensor | None,
+                     ctx_lens: torch.Tensor, tile_req: torch.Tensor | None, tile_tok0: torch.Tensor | None, num_tiles: int,
+                     tile_tokens: int, heads: int, rank: int, rot: int, page_size: int, scale: float, sink: torch.Tensor | None,
+                     splits: int = 1) -> None:
+    """Causal attention of the step's tokens over their requests' cached rows ``plane [pages, 1, page, rank + rot]``: ``q [T,
+    heads * (rank + rot)]`` holds per head the query brought into the cache row's shape, a score is the dot product of the two
+    times ``scale``, the softmax's denominator also holds ``exp(sink[head])`` (float32 ``[heads]``; ``None``: no sink), and ``out
+    [T, heads * rank]`` receives the weighted sums of the rows' first ``rank`` numbers.  ``tile_req = tile_tok0 = None``: every
+    request brings one token.  ``splits``: work-groups that share a tile's keys (merged afterwards)."""
+    T = q.shape[0]
+    D = rank + rot
+    if q.stride(1) != 1 or q.shape[1] < heads * D or out.shape != (T, heads * rank) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("latent_attention: q/out shapes or dtypes do not fit")
+    if plane.dtype != q.dtype or plane.dim() != 4 or tuple(plane.shape[1:]) != (1, page_size, D) or not plane.is_contiguous():
+        raise KernelError(f"latent_attention: plane {tuple(plane.shape)} {plane.dtype} is not [pages, 1, {page_size}, {D}] {q.dtype}")
+    if rank > LATENT_MAX_RANK:
+        raise KernelError(f"latent_attention: built for latents of up to {LATENT_MAX_RANK} numbers")
+    for name, t in (("block_table", block_table), ("ctx_lens", ctx_lens)):
+        _i32(t, name)
+    if tile_req is None:
+        if tile_tok0 is not None or num_tiles != T or ctx_lens.numel() < T or block_table.shape[0] < T:
+            raise KernelError("latent_attention: without a tile list every request brings exactly one token")
+        req_indptr = None
+    else:
+        for name, t in (("req_indptr", req_indptr), ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+            _i32(t, name)
+        if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
+            raise KernelError("latent_attention: tile arrays shorter than the number of tiles")
+    if sink is not None and (sink.dtype != torch.float32 or sink.numel() != heads or not sink.is_contiguous()):
+        raise KernelError("latent_attention: sink must be float32 [heads]")
+    splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * heads * (rank + 2) * 4)))
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((T * heads * splits, rank), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * heads * splits, 2), dtype=torch.float32, device=q.device)
+    lib = _lib("latent")
+    _check(lib, lib.tl_latent_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(plane), _ptr(block_table), c_int(block_table.stride(0)),
+                                        _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T),
+                                        c_int(tile_tokens), c_int(heads), c_int(rank), c_int(rot), c_int(page_size), c_float(scale),
+                                        _ptr(sink), c_int(splits), _ptr(part_o), _ptr(part_ml), c_int(_dt(q, "latent_attention")), _stream()))
+
+
+# ------------------------------------------------------------- products over groups, routing
+
+ACTIVATIONS = {"none": 0, "relu2": 1}
+
+
+def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int) -> None:
+    """Per head ``h``: ``out[:, h * out_head : h * out_head + N] = x[:, h * x_head : h * x_head + K] @ weight[h].T`` with
+    ``weight [heads, N, K]``; ``x`` and ``out`` may be views with longer rows."""
+    G, N, K = weight.shape
+    T = x.shape[0]
+    if x.dtype != weight.dtype or out.dtype != x.dtype or x.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != T or not weight.is_contiguous() \
+            or x.shape[1] < (G - 1) * x_head + K or out.shape[1] < (G - 1) * out_head + N:
+        raise KernelError("heads_linear: shapes or dtypes do not fit")
+    lib = _lib("experts")
+    _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(x_head), c_void_p(0), _ptr(weight), _ptr(out), c_int(out.stride(0)),
+                                    c_int(out_head), c_void_p(0), c_int(G), c_int(T), c_int(N), c_int(K), c_int(0),
+                                    c_int(_dt(x, "heads_linear")), _stream()))
+
+
+def experts_linear(x: torch.Tensor, slot_token: torch.Tensor | None, weight: torch.Tensor, offsets: torch.Tensor, out: torch.Tensor,
+                   activation: str = "none") -> None:
+    """``out[slot] = act(x[row(slot)] @ weight[e].T)`` for the slots ``offsets[e] .. offsets[e + 1] - 1`` of every expert ``e``;
+    ``row(slot)`` is ``slot_token[slot]`` (a token routed to the expert) or, without it, the slot itself.  ``weight [experts, N, K]``,
+    ``out [slots, N]``."""
+    G, N, K = weight.shape
+    S = out.shape[0]
+    if x.dtype != weight.dtype or out.dtype != x.dtype or x.stride(1) != 1 or x.shape[1] != K or out.shape != (S, N) or not out.is_contiguous() \
+            or not weight.is_contiguous() or (slot_token is None and x.shape[0] != S):
+        raise KernelError("experts_linear: shapes or dtypes do not fit")
+    _i32(offsets, "offsets", G + 1)
+    _i32(slot_token, "slot_token", S)
+    lib = _lib("experts")
+    _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(0), _ptr(slot_token), _ptr(weight), _ptr(out), c_int(N), c_int(0),
+                                    _ptr(offsets), c_int(G), c_int(S), c_int(N), c_int(K), c_int(ACTIVATIONS[activation]),
+                                    c_int(_dt(x, "experts_linear")), _stream()))
+
+
+def route(logits: torch.Tensor, top: int):
+    """The ``top`` largest logits of every row of float32 ``logits [T, experts]`` (the lower index wins a tie), the softmax over those
+    alone, and the sort of the (token, choice) pairs by expert: ``(weights [T, top] float32, offsets [experts + 1], slot_token [T * top],
+    pair_slot [T * top])``, all on the GPU: expert ``e`` owns the slots ``offsets[e] .. offsets[e + 1] - 1``, slot ``s`` reads token
+    ``slot_token[s]``, and the output row of token ``t``'s ``j``-th choice is ``pair_slot[t * top + j]``."""
+    T, E = logits.shape
+    if logits.dtype != torch.float32 or not logits.is_contiguous() or not 0 < top <= min(E, 64) or E > 4096:
+        raise KernelError("route: contiguous float32 logits, up to 4096 experts and up to 64 choices")
+    ints = torch.empty(T * top * 3 + E + 1, dtype=torch.int32, device=logits.device)
+    chosen, slot_token, pair_slot, offsets = ints[: T * top], ints[T * top: 2 * T * top], ints[2 * T * top: 3 * T * top], ints[3 * T * top:]
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    lib = _lib("experts")
+    _check(lib, lib.tl_route(_ptr(logits), c_int(T), c_int(E), c_int(top), _ptr(chosen), _ptr(weights), _ptr(offsets), _ptr(slot_token),
+                             _ptr(pair_slot), _stream()))
+    return weights, offsets, slot_token, pair_slot
+
+
+def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = sum_j weights[t, j] * y[pair_slot[t * top + j]]``, summed in 32-bit in the order of the choices."""
+    T, top = weights.shape
+    W = out.shape[1]
+    if y.shape != (T * top, W) or out.shape[0] != T or y.dtype != out.dtype or not y.is_contiguous() or not out.is_contiguous() \
+            or weights.dtype != torch.float32 or not weights.is_contiguous():
+        raise KernelError("combine: shapes or dtypes do not fit")
+    _i32(pair_slot, "pair_slot", T * top)
+    lib = _lib("experts")
+    _check(lib, lib.tl_combine(_ptr(y), _ptr(pair_slot), _ptr(weights), _ptr(out), c_int(T), c_int(top), c_int(W), c_int(_dt(out, "combine")), _stream()))
+
+
+def activation(x: torch.Tensor, kind: str) -> None:
+    """The elementwise activation ``kind`` (``relu2``: the square of relu) on contiguous ``x``, in place."""
+    if not x.is_contiguous():
+        raise KernelError("activation: contiguous tensors only")
+    lib = _lib("experts")
+    _check(lib, lib.tl_activation(_ptr(x), ctypes.c_long(x.numel()), c_int(ACTIVATIONS[kind]), c_int(_dt(x, "activation")), _stream()))

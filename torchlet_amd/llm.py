@@ -232,10 +232,10 @@ def main(argv=None) -> int:
     args = _parser().parse_args(argv)
     if args.command == "init":
         from .engine.loading import parse_dtype
-        from .registry import config_class
+        from .registry import architecture_of, config_class
         from .weights.random_init import write_model_folder
         d = json.loads(Path(args.config).read_text())
-        cfg = config_class(d["architectures"][0]).from_dict(d)
+        cfg = config_class(architecture_of(d, args.config)).from_dict(d)
         folder = write_model_folder(cfg, args.seed, args.out, parse_dtype(args.store_dtype))
         print(folder)
         return 0

@@ -14,7 +14,7 @@ import torch
 from ..config.base import ModelSpec
 from ..kernels import ops
 from ..parts import BLOCKS, NORMS, Stream, WeightSpec
-from ..parts.base import KEEP_COMPUTE, KEEP_STORED, place
+from ..parts.base import KEEP_COMPUTE, KEEP_STORED, join_name, place, under
 
 
 class DecoderModel:
@@ -33,31 +33,28 @@ class DecoderModel:
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> dict[str, WeightSpec]:
         s = self.spec
-        specs = {f"{s.embed_name}.weight": WeightSpec((s.vocab_size, s.hidden))}
+        specs = {join_name(s.embed_name, s.weight_suffix): WeightSpec((s.vocab_size, s.hidden))}
         for i, block in enumerate(self.blocks):
             for k, v in block.weight_specs().items():
-                specs[f"{s.layers_prefix}.{i}.{k}"] = v
+                specs[join_name(s.layer_name(i), k)] = v
         for k, v in self.final_norm.weight_specs().items():
-            specs[f"{s.final_norm_name}.{k}"] = v
+            specs[join_name(s.final_norm_name, k)] = v
         # a tied head is the embedding matrix; a checkpoint may still carry a copy of it
-        specs[f"{s.head_name}.weight"] = WeightSpec((s.vocab_size, s.hidden), optional=s.tie_head)
+        specs[join_name(s.head_name, s.weight_suffix)] = WeightSpec((s.vocab_size, s.hidden), optional=s.tie_head)
         if s.head_bias:
             specs[f"{s.head_name}.bias"] = WeightSpec((s.vocab_size,), keep=KEEP_STORED)
         return specs
 
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
         s = self.spec
-        self.embed = place(tensors[f"{s.embed_name}.weight"], KEEP_COMPUTE, self.dtype, self.device)
-        names = list(tensors)      # `tensors` may read from disk on access: touch each name once
-        for i, block in enumerate(self.blocks):
-            prefix = f"{s.layers_prefix}.{i}."
-            block.load_weights({k[len(prefix):]: tensors[k] for k in names if k.startswith(prefix)})
-        prefix = s.final_norm_name + "."
-        self.final_norm.load_weights({k[len(prefix):]: tensors[k] for k in names if k.startswith(prefix)})
+        self.embed = place(tensors[join_name(s.embed_name, s.weight_suffix)], KEEP_COMPUTE, self.dtype, self.device)
+        for i, block in enumerate(self.blocks):      # (`tensors` may read from disk on access: each name is touched once)
+            block.load_weights(under(tensors, s.layer_name(i)))
+        self.final_norm.load_weights(under(tensors, s.final_norm_name))
         if s.tie_head:
             self.head = self.embed
         else:
-            self.head = place(tensors[f"{s.head_name}.weight"], KEEP_COMPUTE, self.dtype, self.device)
+            self.head = place(tensors[join_name(s.head_name, s.weight_suffix)], KEEP_COMPUTE, self.dtype, self.device)
         if s.head_bias:
             self.head_bias = place(tensors[f"{s.head_name}.bias"], KEEP_STORED, self.dtype, self.device)
 
@@ -86,9 +83,9 @@ class DecoderModel:
 
     def kernel_libraries(self) -> list[str]:
         libs = ["elementwise", "gemm", "sampling"]
-        for b in self.blocks:
-            if hasattr(b.mixer, "kernel_libraries"):
-                libs += b.mixer.kernel_libraries()
+        for part in self.parts():
+            if hasattr(part, "kernel_libraries"):
+                libs += part.kernel_libraries()
         return list(dict.fromkeys(libs))
 
     # ------------------------------------------------------------------ the step

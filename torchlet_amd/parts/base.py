@@ -91,6 +91,19 @@ class WeightSpec:
         return self.keep == KEEP_INT32
 
 
+def join_name(prefix: str, name: str) -> str:
+    """``prefix.name``; a part whose one tensor bears the part's own name declares it as ``""``."""
+    return f"{prefix}.{name}" if name else prefix
+
+
+def under(tensors, prefix: str) -> dict:
+    """The tensors of the part called ``prefix``, by the names the part declared them with (``""`` for ``prefix`` itself)."""
+    out = {k[len(prefix) + 1:]: tensors[k] for k in list(tensors) if k.startswith(prefix + ".")}
+    if prefix in tensors:
+        out[""] = tensors[prefix]
+    return out
+
+
 def place(t: torch.Tensor, keep: str, dtype: torch.dtype, device) -> torch.Tensor:
     """``t`` on ``device`` in the dtype that the policy ``keep`` gives it under an engine of ``dtype``."""
     if keep not in DTYPE_POLICIES:
@@ -175,11 +188,12 @@ class Stream:
     over the residual per branch.  ``pending`` is ``[T, hidden]`` in the activation dtype, or
     float32 ``[P, T, hidden]``: P slabs of partial sums that the norm adds up as well."""
 
-    __slots__ = ("residual", "pending")
+    __slots__ = ("residual", "pending", "normed")
 
     def __init__(self, residual: torch.Tensor, pending: torch.Tensor | None = None):
         self.residual = residual
         self.pending = pending
+        self.normed = None      # blocks whose norm follows the sum: the residual in the activation dtype, as the last norm left it
 
 
 class LazyNorm:
@@ -229,6 +243,11 @@ class Norm(Part):
         return ``norm(residual) * gain`` in the activation dtype (the factor applied in 32-bit, before
         the one rounding of the result).  With ``rows`` (int32 indices) only those rows are read
         and returned, and the stream is left untouched."""
+        raise NotImplementedError
+
+    def renorm(self, stream: Stream, alpha: float = 1.0) -> torch.Tensor:
+        """The norm after the sum: ``stream.residual <- norm(alpha * residual + pending)`` in 32-bit (the pending branch is
+        used up), returned in the activation dtype as well, for the next sublayer to read."""
         raise NotImplementedError
 
     def lazy(self, stream: Stream) -> "LazyNorm | None":

@@ -1,0 +1,103 @@
+"""Feed-forward layers with an elementwise activation: a dense one with biases, and a mixture of experts.
+
+Dense: ``W_down act(W_up h + b_up) + b_down``.  Routed: the router's logits ``z = W_r h + b_r`` leave their product in
+32-bit (the operands are ``h`` as the stream's norm rounded it and the router's matrix as stored, so the products are
+exact and the sums 32-bit); per token the ``top`` largest are chosen (the lower index wins a tie), their softmax (over
+the chosen ones alone, in 32-bit) weighs the experts' outputs ``W_down,e act(W_up,e h)``, which are summed in the order
+of the choices.  The choice, the sort of the (token, choice) pairs by expert and the products over the experts' rows all
+happen on the GPU from device-side counts: nothing of a step's routing is read on the host, so decode steps can be
+recorded as graphs.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import ops
+from .base import FEED_FORWARDS, KEEP_COMPUTE, KEEP_FLOAT32, FeedForward, WeightSpec
+
+
+def _activation(name: str) -> str:
+    if name not in ops.ACTIVATIONS:
+        raise ConfigError(f"no activation {name!r}; built: {', '.join(sorted(ops.ACTIVATIONS))}")
+    return name
+
+
+@FEED_FORWARDS.register("dense_ff")
+class DenseFF(FeedForward):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.hidden, self.inter, self.act = spec.hidden, spec.intermediate, _activation(spec.activation)
+        self.w_up = self.b_up = self.w_down = self.b_down = None
+
+    def kernel_libraries(self):
+        return ["experts"]
+
+    def weight_specs(self):
+        specs = {"up": WeightSpec((self.inter, self.hidden)), "down": WeightSpec((self.hidden, self.inter))}
+        if self.spec.bias:
+            specs["up.b"] = WeightSpec((self.inter,), keep=KEEP_FLOAT32)
+            specs["down.b"] = WeightSpec((self.hidden,), keep=KEEP_FLOAT32)
+        return specs
+
+    def load_weights(self, tensors):
+        self.w_up = self._place(tensors["up"], KEEP_COMPUTE)
+        self.w_down = self._place(tensors["down"], KEEP_COMPUTE)
+        if self.spec.bias:
+            self.b_up = self._place(tensors["up.b"], KEEP_FLOAT32)
+            self.b_down = self._place(tensors["down.b"], KEEP_FLOAT32)
+
+    def forward(self, h, ctx):
+        T = h.shape[0]
+        z = torch.empty((T, self.inter), dtype=self.dtype, device=h.device)
+        ops.linear(h, self.w_up, self.b_up, z)
+        ops.activation(z, self.act)
+        y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
+        ops.linear(z, self.w_down, self.b_down, y)
+        return y
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if not 0 < spec.top <= spec.experts:
+            raise ConfigError(f"a router picks between 1 and all of its experts, not {spec.top} of {spec.experts}")
+        self.hidden, self.inter, self.experts, self.top = spec.hidden, spec.intermediate, spec.experts, spec.top
+        self.act = _activation(spec.activation)
+        self.w_router = self.b_router = self.w_up = self.w_down = None
+
+    def kernel_libraries(self):
+        return ["experts"]
+
+    def weight_specs(self):
+        specs = {"router": WeightSpec((self.experts, self.hidden))}
+        if self.spec.router_bias:
+            specs["router.b"] = WeightSpec((self.experts,), keep=KEEP_FLOAT32)
+        for e in range(self.experts):
+            specs[f"e{e}.up"] = WeightSpec((self.inter, self.hidden))
+            specs[f"e{e}.down"] = WeightSpec((self.hidden, self.inter))
+        return specs
+
+    def load_weights(self, tensors):
+        self.w_router = self._place(tensors["router"], KEEP_COMPUTE)
+        self.b_router = self._place(tensors["router.b"], KEEP_FLOAT32) if self.spec.router_bias else None
+        self.w_up = self._place(torch.stack([tensors[f"e{e}.up"] for e in range(self.experts)]), KEEP_COMPUTE)
+        self.w_down = self._place(torch.stack([tensors[f"e{e}.down"] for e in range(self.experts)]), KEEP_COMPUTE)
+
+    def forward(self, h, ctx):
+        T = h.shape[0]
+        logits = torch.empty((T, self.experts), dtype=torch.float32, device=h.device)
+        ops.linear(h, self.w_router, self.b_router, logits)
+        weights, offsets, slot_token, pair_slot = ops.route(logits, self.top)
+        z = torch.empty((T * self.top, self.inter), dtype=self.dtype, device=h.device)
+        ops.experts_linear(h, slot_token, self.w_up, offsets, z, self.act)
+        y = torch.empty((T * self.top, self.hidden), dtype=self.dtype, device=h.device)
+        ops.experts_linear(z, None, self.w_down, offsets, y)
+        out = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
+        ops.combine(y, pair_slot, weights, out)
+        return out

@@ -1,0 +1,117 @@
+"""Attention over a cached latent, with a sink in the softmax.
+
+Queries come through a latent: ``c_q = rmsnorm(W_dq h) * w_dq``, ``q = W_uq c_q``, per head ``dim`` unrotated and
+``rot_dim`` rotated numbers.  ``W_dkv h`` gives ``kv_rank`` numbers whose norm ``c = rmsnorm(.) * w_dkv`` is the token's
+latent, and ``rot_dim`` more that are one rotated key part shared by all heads.  Per head the unrotated key is ``W_uk c``
+and the value ``W_uv c``; the score of query ``t`` and key ``s <= t`` is ``(q_t . k_s + q_t^rot . k_s^rot) * scale``, the
+softmax's denominator also holds ``exp(sink_head)`` (a term without key or value), and ``W_o`` follows on the heads' values.
+
+Only ``c`` and the rotated key part are cached: one page plane whose rows hold ``kv_rank + rot_dim`` numbers.  The key
+up-projection is taken to the query's side, ``q_t . (W_uk c_s) = (W_uk^T q_t) . c_s``, so a head's query becomes a vector
+of the cache row's shape and all heads read the same rows: the attention kernel is one dot product per key and its
+weighted sum runs over the latents; the value up-projection ``W_uv`` is applied to that sum.  Prompts and decode steps
+take the same path, so how a request is cut cannot change what it computes beyond the order of the sums.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import ops
+from .base import KEEP_COMPUTE, KEEP_FLOAT32, KEEP_STORED, MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
+
+_MIN_KEYS_PER_SPLIT = 128
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.kv_rank > ops.LATENT_MAX_RANK:
+            raise ConfigError(f"latent attention is built for latents of up to {ops.LATENT_MAX_RANK} numbers, not {spec.kv_rank}")
+        self.hidden, self.heads = spec.hidden, spec.heads
+        self.dim, self.rot, self.vdim, self.rank, self.q_rank = spec.dim, spec.rot_dim, spec.vdim, spec.kv_rank, spec.q_rank
+        self.row = spec.kv_rank + spec.rot_dim               # numbers of a cache row, and of a head's query against it
+        self.scale = float(spec.scale)
+        self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
+        if self.position is not None and not hasattr(self.position, "inv_freq"):
+            raise ConfigError("latent attention folds a rotation in pairs into its kernels; its position encoding must offer inv_freq")
+        self.tile_tokens = ops.latent_tile_tokens(self.heads)
+        self.compute_units = ops.compute_units()
+        self.w_down = self.w_dq_norm = self.w_dkv_norm = self.w_uq = self.w_uk_t = self.w_uv = self.sink = self.w_o = None
+
+    def paged_need(self):
+        return PagedNeed(num_heads=1, head_dim=self.row, planes=((1, self.row),))
+
+    def kernel_libraries(self):
+        return ["latent", "experts"]
+
+    def parts(self):
+        yield self
+        if self.position is not None:
+            yield from self.position.parts()
+
+    def weight_specs(self):
+        H, n = self.hidden, self.heads
+        specs = {
+            "dq": WeightSpec((self.q_rank, H)), "dq.norm": WeightSpec((self.q_rank,), keep=KEEP_STORED, init="one_plus_normal"),
+            "uq": WeightSpec((n * (self.dim + self.rot), self.q_rank)),
+            "dkv": WeightSpec((self.row, H)), "dkv.norm": WeightSpec((self.rank,), keep=KEEP_STORED, init="one_plus_normal"),
+            "uk": WeightSpec((n * self.dim, self.rank)), "uv": WeightSpec((n * self.vdim, self.rank)),
+            "o": WeightSpec((H, n * self.vdim)),
+        }
+        if self.spec.sink:
+            specs["sink"] = WeightSpec((n,), keep=KEEP_FLOAT32)
+        return specs
+
+    def load_weights(self, tensors):
+        n = self.heads
+        self.w_down = self._place(torch.cat((tensors["dq"], tensors["dkv"]), dim=0), KEEP_COMPUTE)    # one product reads h once
+        self.w_dq_norm = self._place(tensors["dq.norm"], KEEP_STORED)
+        self.w_dkv_norm = self._place(tensors["dkv.norm"], KEEP_STORED)
+        self.w_uq = self._place(tensors["uq"], KEEP_COMPUTE)
+        # per head the key up-projection transposed, [rank, dim]: it multiplies the unrotated query
+        self.w_uk_t = self._place(tensors["uk"].view(n, self.dim, self.rank).transpose(1, 2).contiguous(), KEEP_COMPUTE)
+        self.w_uv = self._place(tensors["uv"].view(n, self.vdim, self.rank).contiguous(), KEEP_COMPUTE)
+        self.sink = self._place(tensors["sink"], KEEP_FLOAT32) if self.spec.sink else None
+        self.w_o = self._place(tensors["o"], KEEP_COMPUTE)
+
+    def _splits(self, ctx, tiles: int) -> int:
+        """Work-groups that share a tile's keys: enough to give every compute unit one, no part under 128 keys."""
+        groups = max(1, tiles * -(-self.heads // ops.LATENT_ATTENTION_ROWS))
+        return max(1, min(self.compute_units // groups, ctx.max_total_len // _MIN_KEYS_PER_SPLIT, 32))
+
+    def forward(self, h, ctx, cache):
+        T, n = h.shape[0], self.heads
+        dev = h.device
+        inv_freq = self.position.inv_freq if self.position is not None else torch.zeros(0, dtype=torch.float32, device=dev)
+        rot_dims = 2 * inv_freq.numel()
+        plane = cache.planes[0]
+        table = ctx.block_tables[cache.group]
+        down = torch.empty((T, self.q_rank + self.row), dtype=self.dtype, device=dev)
+        ops.linear(h, self.w_down, None, down)
+        cq = torch.empty((T, self.q_rank), dtype=self.dtype, device=dev)
+        write = (ctx.token_req, table, plane, cache.page_size) if cache.writable else (None, None, None, 0)
+        ops.latent_prepare(down, self.q_rank, self.rank, self.rot, rot_dims, self.w_dq_norm, self.w_dkv_norm, float(self.spec.norm_eps),
+                           ctx.positions, inv_freq, cq, *write)
+        q = torch.empty((T, n * (self.dim + self.rot)), dtype=self.dtype, device=dev)
+        ops.linear(cq, self.w_uq, None, q)
+        # the query against a cache row: [W_uk^T q_unrotated, rotated part], head by head
+        qrow = torch.empty((T, n * self.row), dtype=self.dtype, device=dev)
+        ops.heads_linear(q, self.dim + self.rot, self.w_uk_t, qrow, self.row)
+        ops.rotate_pairs(q, self.dim + self.rot, self.dim, qrow, self.row, self.rank, ctx.positions, inv_freq, n, self.rot)
+        tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
+        if ctx.decode_only and tiles == T:          # one token per request: no tile list to look up
+            tile_req = tile_tok0 = None
+        mixed_latent = torch.empty((T, n * self.rank), dtype=self.dtype, device=dev)
+        ops.latent_attention(qrow, mixed_latent, plane, table, ctx.req_indptr, ctx.ctx_lens, tile_req, tile_tok0, tiles, self.tile_tokens,
+                             n, self.rank, self.rot, cache.page_size, self.scale, self.sink, self._splits(ctx, tiles))
+        values = torch.empty((T, n * self.vdim), dtype=self.dtype, device=dev)
+        ops.heads_linear(mixed_latent, self.rank, self.w_uv, values, self.vdim)
+        if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, n * self.vdim):
+            return ops.linear_partials(values, self.w_o)      # few rows against a narrow matrix: the next norm adds the slabs up
+        out = torch.empty((T, self.hidden), dtype=self.dtype, device=dev)
+        ops.linear(values, self.w_o, None, out)
+        return out

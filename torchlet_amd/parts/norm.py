@@ -24,10 +24,10 @@ class RMSNorm(Norm):
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.dim,), keep=KEEP_STORED, init="one_plus_normal")}
+        return {self.spec.weight_name: WeightSpec((self.dim,), keep=KEEP_STORED, init="one_plus_normal")}
 
     def load_weights(self, tensors):
-        self.weight = self._place(tensors["weight"], KEEP_STORED)
+        self.weight = self._place(tensors[self.spec.weight_name], KEEP_STORED)
 
     def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
         n = stream.residual.shape[0] if rows is None else rows.numel()
@@ -35,6 +35,16 @@ class RMSNorm(Norm):
         ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, out, rows, gain)
         if rows is None:
             stream.pending = None
+        return out
+
+    def renorm(self, stream: Stream, alpha: float = 1.0) -> torch.Tensor:
+        if self.dtype == torch.float32:              # the residual itself is what the next sublayer reads
+            ops.scaled_add_rmsnorm(stream.residual, stream.pending, alpha, self.weight, self.eps, None)
+            stream.pending = None
+            return stream.residual
+        out = torch.empty(stream.residual.shape, dtype=self.dtype, device=stream.residual.device)
+        ops.scaled_add_rmsnorm(stream.residual, stream.pending, alpha, self.weight, self.eps, out)
+        stream.pending = None
         return out
 
     def lazy(self, stream: Stream) -> LazyNorm | None:

@@ -39,3 +39,28 @@ class RotaryEncoding(PositionEncoding):
             T, heads, hd = x.shape
             flat = x.as_strided((T, heads * hd), (x.stride(0), 1))
             ops.rope_cache_write(flat, heads, 0, hd, heads, positions, self.inv_freq)
+
+
+@POSITION_ENCODINGS.register("rope_pairs")
+class PairRotaryEncoding(PositionEncoding):
+    """The interleaved layout: of the first ``dims`` entries of a vector, entry ``2i`` is paired with ``2i + 1`` and the pair
+    ``(u, v)`` at position ``p`` becomes ``(u cos a - v sin a, v cos a + u sin a)`` with ``a = float32(p) * f_i``,
+    ``f_i = base**(-2i / dims)`` (taken in 64-bit on the host, then rounded once to 32-bit); entries beyond ``dims`` pass
+    unchanged.  Mixers fold the rotation into their own kernels through :attr:`inv_freq`; :meth:`apply` turns whole heads."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.dims % 2 or spec.dims <= 0:
+            raise ConfigError(f"rotary encoding in pairs needs an even, positive number of dimensions, got {spec.dims}")
+        self.dims = spec.dims
+        i = torch.arange(spec.dims // 2, dtype=torch.float64)
+        self.inv_freq = (float(spec.base) ** (-2.0 * i / spec.dims)).to(torch.float32).to(device)
+
+    def apply(self, q, k, positions):
+        for x in (q, k):
+            if x is None:
+                continue
+            T, heads, hd = x.shape
+            flat = x.as_strided((T, heads * hd), (x.stride(0), 1))
+            ops.rotate_pairs(flat, hd, 0, flat, hd, 0, positions, self.inv_freq, heads, hd)

@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (``config.json``'s ``architectures[0]``) to
+"""One registry from an architecture's name (``config.json``'s ``architectures[0]``, or its ``architecture``) to
 its typed configuration.  A configuration expands into a model specification, and every
 architecture is run by the same :class:`~torchlet_amd.models.decoder.DecoderModel`, so
 adding an architecture means adding a configuration class (and parts, if it needs new ones).
@@ -9,6 +9,7 @@ import json
 from pathlib import Path
 
 from .config.base import ConfigError, ModelConfig
+from .config.migurax import MiguraxConfig
 from .config.qwen2 import Qwen2Config
 
 ARCHITECTURES: dict[str, type[ModelConfig]] = {}
@@ -26,6 +27,7 @@ def unregister_architecture(name: str) -> None:
 
 
 register_architecture(Qwen2Config)
+register_architecture(MiguraxConfig)
 
 
 def config_class(name: str) -> type[ModelConfig]:
@@ -41,7 +43,14 @@ def load_config(folder: str | Path) -> ModelConfig:
     if not path.exists():
         raise FileNotFoundError(f"no config.json in {folder}")
     d = json.loads(path.read_text())
+    return config_class(architecture_of(d, str(path))).from_dict(d)
+
+
+def architecture_of(d: dict, where: str = "config.json") -> str:
+    """The architecture a ``config.json`` names: the first entry of its list ``architectures``, or its string ``architecture``."""
     archs = d.get("architectures")
-    if not isinstance(archs, list) or not archs:
-        raise ConfigError(f"{path}: 'architectures' must be a non-empty list")
-    return config_class(archs[0]).from_dict(d)
+    if isinstance(archs, list) and archs:
+        return archs[0]
+    if isinstance(d.get("architecture"), str) and d["architecture"]:
+        return d["architecture"]
+    raise ConfigError(f"{where}: 'architectures' must be a non-empty list (or 'architecture' a name)")
