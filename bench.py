@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
                     [--shape 7b|14b|32b] [--context N] [--new-tokens G] [--prefill-tokens T]
-                    [--workload decode|serve] [--only decode|step|prefill] [--all]
+                    [--workload decode|serve|migurax] [--only decode|step|prefill] [--all]
 
 The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV heads, head
 size 128, intermediate 18944, vocabulary 152064) with random weights and goes through the whole engine
@@ -32,6 +32,13 @@ with 4096-token prompts (``decode_32b_b16_ctx4096``), each with the bare step fu
 second figure (``step_function``), and the prefill of 16384 tokens as steps of the step function alone; and the same
 32B sizes in true 32-bit, all 64 layers (``fp32_32b``: decode at batch 1 through the engine, prefill of 2048 tokens).
 ``--workload serve`` prints the serving run alone as a line of its own.
+
+``--workload migurax [--size s|m]`` prints a line of its own for the Migurax design (post-norm layers with a matrix-memory
+recurrence or attention over a cached latent, dense or routed feed-forwards) at layer sizes that resemble a real model's,
+with random weights: prefill of ``--prefill-tokens`` tokens in one step and decode steps at ``--batch`` on ``--context``-token
+caches (replayed graphs), beside a Qwen2 model of the same width, layer count and dense feed-forward width; and, under
+``kernels``, every kernel that is the design's own alone at those sizes beside the like kernel of the Qwen2 path, each with
+the bytes it must move or the operations it must do and the fraction of the GPU's rate that this makes.
 """
 from __future__ import annotations
 
@@ -74,7 +81,8 @@ def parse_args(argv=None):
     p.add_argument("--context", type=int, default=CONTEXT, help="prompt tokens of each request in the decode runs")
     p.add_argument("--new-tokens", type=int, default=None, help="tokens each request may generate (decode: 256, serve: 128)")
     p.add_argument("--prefill-tokens", type=int, default=2048)
-    p.add_argument("--workload", choices=["decode", "serve"], default="decode")
+    p.add_argument("--workload", choices=["decode", "serve", "migurax"], default="decode")
+    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax: layer sizes (s: width 2048, m: width 4096)")
     p.add_argument("--requests", type=int, default=32)
     p.add_argument("--prompt-min", type=int, default=128)
     p.add_argument("--prompt-max", type=int, default=4096)
@@ -469,6 +477,231 @@ def prefill_flops_step(cfg, tokens: int, context: int) -> float:
     return 2.0 * tokens * linear + attn
 
 
+# ---------------------------------------------------------------------------------------------- the Migurax design
+
+def _latent_layer(heads, dim, rot, vdim, rank, q_rank, mlp):
+    return dict(type="latent_attention", mlp=mlp, mixer=dict(heads=heads, dim=dim, rot_dim=rot, vdim=vdim, kv_rank=rank, q_rank=q_rank,
+                                                             scale=(dim + rot) ** -0.5, rot=dict(base=10000.0, dims=rot)))
+
+
+def migurax_sizes(size: str) -> tuple[dict, dict]:
+    """A Migurax configuration of four layers (recurrence + dense, latent attention + routed twice, recurrence + routed) and the
+    Qwen2 configuration of the same width, layer count, vocabulary and dense feed-forward width."""
+    width, heads, ff, experts, eff, top, q_rank, mheads = dict(s=(2048, 16, 8192, 16, 1024, 2, 768, 4), m=(4096, 32, 16384, 32, 2048, 4, 1536, 8))[size]
+    moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, top=top))
+    rec = dict(heads=mheads, dim=256, vdim=512, gate_cap=15.0)
+    layers = [dict(type="mlstm", mixer=rec, mlp=dict(kind="dense", ff=ff)), _latent_layer(heads, 128, 64, 128, 512, q_rank, moe),
+              _latent_layer(heads, 128, 64, 128, 512, q_rank, moe), dict(type="mlstm", mixer=rec, mlp=moe)]
+    ours = dict(architecture="Migurax", vocab=32000, width=width, postln_alpha=1.0, norm=dict(eps=1e-5), layers=layers, max_positions=8192)
+    like = dict(QWEN25_7B, vocab_size=32000, hidden_size=width, num_hidden_layers=4, num_attention_heads=heads, num_key_value_heads=heads // 4,
+                intermediate_size=ff * 2 // 3 // 256 * 256, max_position_embeddings=8192)      # three matrices of 2/3 the width: as many weights as two
+    return ours, like
+
+
+def _build_from(d: dict, dtype: str):
+    import torch
+    from torchlet_amd.engine.loading import build_model
+    from torchlet_amd.registry import architecture_of, config_class
+    from torchlet_amd.weights.random_init import RandomTensors
+    cfg = config_class(architecture_of(d)).from_dict(d)
+    model = build_model(cfg, dtype, tensors=RandomTensors(cfg, seed=2, dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32, device="cuda"))
+    torch.cuda.empty_cache()
+    return cfg, model
+
+
+def _decode_ms(model, batch: int, steps: int, warmup: int, context: int) -> float:
+    """ms of a decode step of the bare step function (replayed graphs, tokens taken on the GPU from the sampling of the step
+    before) on caches of ``context`` tokens with random contents."""
+    import torch
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import make_runner
+    from torchlet_amd.sampling.sampler import Sampler
+    runner = make_runner(model, page_size=PAGE, num_pages=batch * (-(-(context + steps + warmup + 2) // PAGE)) + 1, max_requests=batch, use_graphs=True)
+    ids = [f"b{i}" for i in range(batch)]
+    fill_context(runner, ids, context)
+    sampler, zeros = Sampler(0), [0.0] * batch
+    drawn = sampler.launch(runner.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids)]), zeros, zeros, zeros)
+    entries = [StepEntry(r, [0], [0]) for r in ids]
+
+    def step():
+        nonlocal drawn
+        drawn = sampler.launch(runner.step(entries, device_tokens=(drawn.device, None)), zeros, zeros, zeros)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    assert runner.graph_replays >= steps or not runner.use_graphs
+    del runner
+    torch.cuda.empty_cache()
+    return ms
+
+
+def _weight_bytes(model) -> int:
+    """Bytes of every tensor a model's parts hold on the GPU (what a decode step reads at most of them)."""
+    import torch
+    seen, total = set(), 0
+    for part in list(model.parts()) + [model]:
+        for v in vars(part).values():
+            if isinstance(v, torch.Tensor) and v.is_cuda and v.data_ptr() not in seen:
+                seen.add(v.data_ptr())
+                total += v.numel() * v.element_size()
+    return total
+
+
+def migurax_kernels(ours: dict, like: dict, batch: int, context: int, tokens: int) -> list[dict]:
+    """Each kernel that is the design's own, alone, at the sizes of ``ours``, in a decode step of ``batch`` requests on ``context``
+    cached tokens and in a prompt of ``tokens`` tokens, beside the like kernel of the Qwen2 path at the sizes of ``like``.  ``frac``:
+    bytes that must move / time against 8 TB/s, or operations / time against the matrix cores' bfloat16 rate (against the 32-bit
+    vector rate for the recurrence, which the design wants in 32-bit)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, kind, launch, nbytes=0.0, flops=0.0, peak=MFMA_PEAK_TFLOPS["bfloat16"]):
+        ms = _best_ms(launch, rounds=3, calls=5)
+        row = {"kernel": name, "like": kind, "ms": round(ms, 4)}
+        if nbytes:
+            row.update(bytes=int(nbytes), frac=round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), bound="hbm")
+        else:
+            row.update(flops=flops, frac=round(flops / (ms * 1e-3) / (peak * 1e12), 4), bound="flops")
+        rows.append(row)
+        say(f"  {name}: {ms:.4f} ms, {row['frac']} of its bound")
+
+    def tables(n_req, total):
+        blocks = -(-total // PAGE)
+        table = (torch.arange(n_req * blocks, dtype=torch.int32, device=dev) + 1).view(n_req, blocks)
+        return table, n_req * blocks + 1
+
+    rec = ours["layers"][0]["mixer"]
+    lat = ours["layers"][1]["mixer"]
+    moe = ours["layers"][1]["mlp"]
+    width = ours["width"]
+    # ---- the recurrence: a decode step reads and writes every state once; a prompt does 4 operations per state element and token
+    h, d, v = rec["heads"], rec["dim"], rec["vdim"]
+    for name, T, reqs in (("mlstm_scan decode", batch, batch), (f"mlstm_scan prompt {tokens}", tokens, 1)):
+        qkv = torch.randn(T, 2 * h * d + 2 * h * v, device=dev).to(bf)
+        gates = torch.randn(T, 2 * h, device=dev)
+        state = torch.zeros(reqs + 1, h, d * v + d + 1, device=dev)
+        out = torch.empty(T, h * v, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        launch = lambda: ops.mlstm_scan(qkv, h * d, 2 * h * d, gates, state, slots, indptr, out, h, d, v, 15.0, d ** -0.5, 1e-6)
+        if reqs > 1:
+            add(name, "paged_attention decode", launch, nbytes=2.0 * reqs * h * d * v * 4)
+        else:
+            add(name, "paged_attention_prompt", launch, flops=4.0 * T * h * d * v, peak=MFMA_PEAK_TFLOPS["float32"])
+    # ---- the latent attention: a decode step reads every cached row once; a prompt's scores and sums
+    H, R, rot = lat["heads"], lat["kv_rank"], lat["rot_dim"]
+    D = R + rot
+    sink = torch.zeros(H, device=dev)
+    for name, T, reqs, ctx in (("latent_attention decode", batch, batch, context), (f"latent_attention prompt {tokens}", tokens, 1, 0)):
+        total = ctx + T // reqs
+        table, pages = tables(reqs, total)
+        plane = (torch.randn(pages, 1, PAGE, D, device=dev) * 0.3).to(bf)
+        q = (torch.randn(T, H * D, device=dev) * 0.3).to(bf)
+        out = torch.empty(T, H * R, dtype=bf, device=dev)
+        ctx_lens = torch.full((reqs,), ctx, dtype=torch.int32, device=dev)
+        tq = ops.latent_tile_tokens(H)
+        if reqs > 1:
+            launch = lambda: ops.latent_attention(q, out, plane, table, None, ctx_lens, None, None, T, tq, H, R, rot, PAGE, 0.07, sink,
+                                                  max(1, min(ops.compute_units() // max(1, T * -(-H // 16)), total // 128, 32)))
+            add(name, "paged_attention decode", launch, nbytes=float(reqs) * total * D * 2)
+        else:
+            tiles = -(-T // tq)
+            tile_req = torch.zeros(tiles, dtype=torch.int32, device=dev)
+            tile_tok0 = torch.arange(tiles, dtype=torch.int32, device=dev) * tq
+            indptr = torch.tensor([0, T], dtype=torch.int32, device=dev)
+            launch = lambda: ops.latent_attention(q, out, plane, table, indptr, ctx_lens, tile_req, tile_tok0, tiles, tq, H, R, rot, PAGE, 0.07, sink, 1)
+            add(name, "paged_attention_prompt", launch, flops=float(H) * (2 * D + 2 * R) * T * T / 2)
+    # ---- the products over heads (query onto the latent, values from the latent) and over experts
+    for name, T in (("heads_linear decode", batch), (f"heads_linear prompt {tokens}", tokens)):
+        x = torch.randn(T, H * (lat["dim"] + rot), device=dev).to(bf)
+        w = torch.randn(H, R, lat["dim"], device=dev).to(bf)
+        out = torch.empty(T, H * D, dtype=bf, device=dev)
+        launch = lambda: ops.heads_linear(x, lat["dim"] + rot, w, out, D)
+        if T == batch:
+            add(name, "linear (few rows)", launch, nbytes=float(w.numel()) * 2)
+        else:
+            add(name, "linear (many rows)", launch, flops=2.0 * T * H * R * lat["dim"])
+    E, top, ff = moe["router"]["experts"], moe["router"]["top"], moe["expert"]["ff"]
+    for name, T in (("experts_linear decode", batch), (f"experts_linear prompt {tokens}", tokens)):
+        x = torch.randn(T, width, device=dev).to(bf)
+        w_up = (torch.randn(E, ff, width, device=dev) * 0.02).to(bf)
+        logits = torch.randn(T, E, device=dev)
+        weights, offsets, slot_token, pair_slot = ops.route(logits, top)
+        z = torch.empty(T * top, ff, dtype=bf, device=dev)
+        launch = lambda: ops.experts_linear(x, slot_token, w_up, offsets, z, "relu2")
+        if T == batch:
+            add(name, "linear (few rows)", launch, nbytes=float(min(E, T * top)) * ff * width * 2)
+        else:
+            add(name, "linear (many rows)", launch, flops=2.0 * T * top * ff * width)
+    # ---- the like kernels of the Qwen2 path at the like sizes
+    qh, kvh, hd = like["num_attention_heads"], like["num_key_value_heads"], 128
+    table, pages = tables(batch, context + 1)
+    k_plane = (torch.randn(pages, kvh, PAGE, hd, device=dev) * 0.3).to(bf)
+    v_plane = (torch.randn(pages, kvh, hd, PAGE, device=dev) * 0.3).to(bf)
+    q = (torch.randn(batch, qh * hd, device=dev) * 0.3).to(bf)
+    out = torch.empty(batch, qh * hd, dtype=bf, device=dev)
+    ctx_lens = torch.full((batch,), context, dtype=torch.int32, device=dev)
+    add("paged_attention decode (Qwen2 path)", "", lambda: ops.paged_attention(q, out, k_plane, v_plane, table, None, ctx_lens, None, None, batch, ops.attention_tile_tokens(qh, kvh), qh, kvh, hd, PAGE,
+                                                                              0, hd ** -0.5, 8, waves=8), nbytes=2.0 * batch * (context + 1) * kvh * hd * 2)
+    table, pages = tables(1, tokens)
+    k_plane = (torch.randn(pages, kvh, PAGE, hd, device=dev) * 0.3).to(bf)
+    v_plane = (torch.randn(pages, kvh, hd, PAGE, device=dev) * 0.3).to(bf)
+    q = (torch.randn(tokens, qh * hd, device=dev) * 0.3).to(bf)
+    out = torch.empty(tokens, qh * hd, dtype=bf, device=dev)
+    tq = ops.prompt_attention_tile_tokens(qh, kvh)
+    tiles = -(-tokens // tq)
+    tile_req = torch.zeros(tiles, dtype=torch.int32, device=dev)
+    tile_tok0 = torch.arange(tiles, dtype=torch.int32, device=dev) * tq
+    indptr = torch.tensor([0, tokens], dtype=torch.int32, device=dev)
+    zero = torch.zeros(1, dtype=torch.int32, device=dev)
+    add(f"paged_attention_prompt {tokens} (Qwen2 path)", "", lambda: ops.paged_attention_prompt(q, out, k_plane, v_plane, table, indptr, zero, tile_req, tile_tok0, tiles, tq,
+                                                                                                qh, kvh, hd, PAGE, 0, hd ** -0.5, max_total_len=tokens),
+        flops=float(qh) * 4 * hd * tokens * tokens / 2)
+    inter = like["intermediate_size"]
+    for name, T in (("linear decode (Qwen2 path, down projection)", batch), (f"linear prompt {tokens} (Qwen2 path, down projection)", tokens)):
+        x = torch.randn(T, inter, device=dev).to(bf)
+        w = (torch.randn(width, inter, device=dev) * 0.02).to(bf)
+        out = torch.empty(T, width, dtype=bf, device=dev)
+        launch = lambda: ops.linear(x, w, None, out)
+        if T == batch:
+            add(name, "", launch, nbytes=float(w.numel()) * 2)
+        else:
+            add(name, "", launch, flops=2.0 * T * width * inter)
+    return rows
+
+
+def migurax(args) -> dict:
+    import torch
+    ours, like = migurax_sizes(args.size)
+    out = {"metric": f"Migurax design, size {args.size} (width {ours['width']}, 4 layers), prefill of {args.prefill_tokens} tokens and decode at batch "
+                     f"{args.batch} on {args.context}-token caches, beside Qwen2 sizes of equal width, one MI355X",
+           "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: seeded random weights, token ids and cache contents", "config": {"migurax": ours, "qwen2": like}}
+    for key, d in (("migurax", ours), ("qwen2", like)):
+        say(f"building the {key} model")
+        cfg, model = _build_from(d, args.dtype)
+        pms, pbest = time_prefill(model, args.prefill_tokens)
+        dms = _decode_ms(model, args.batch, min(args.steps, 64), args.warmup, args.context)
+        out[key] = {"weight_bytes": _weight_bytes(model),
+                    "prefill": {"tokens": args.prefill_tokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "tokens_per_s": round(args.prefill_tokens * 1e3 / pms, 1)},
+                    "decode": {"batch": args.batch, "context": args.context, "ms_per_step": round(dms, 4), "tokens_per_s": round(args.batch * 1e3 / dms, 1)}}
+        say(f"{key}: {out[key]}")
+        del model
+        torch.cuda.empty_cache()
+    out["value"] = out["migurax"]["decode"]["tokens_per_s"]
+    if args.dtype == "bfloat16" and not args.no_points:
+        out["kernels"] = migurax_kernels(ours, like, args.batch, args.context, args.prefill_tokens)
+    return out
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     args.serve_new_tokens = args.new_tokens or 128
@@ -480,6 +713,9 @@ def main(argv=None) -> int:
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X; no GPU is visible", file=sys.stderr)
         return 1
+    if args.workload == "migurax":
+        print(json.dumps(migurax(args)))
+        return 0
     name, sizes = SHAPES[args.shape]
     full_layers = sizes["num_hidden_layers"]
     layers = args.layers if args.layers is not None else full_layers
