@@ -607,10 +607,10 @@ def migurax_kernels(ours: dict, like: dict, batch: int, context: int, tokens: in
         q = (torch.randn(T, H * D, device=dev) * 0.3).to(bf)
         out = torch.empty(T, H * R, dtype=bf, device=dev)
         ctx_lens = torch.full((reqs,), ctx, dtype=torch.int32, device=dev)
-        tq = ops.latent_tile_tokens(H)
+        tq = ops.latent_tile_tokens(H, ops.LATENT_MFMA_ROWS if ops.latent_attention_mfma_fits(bf, H, R, rot) else ops.LATENT_ATTENTION_ROWS)
         if reqs > 1:
             launch = lambda: ops.latent_attention(q, out, plane, table, None, ctx_lens, None, None, T, tq, H, R, rot, PAGE, 0.07, sink,
-                                                  max(1, min(ops.compute_units() // max(1, T * -(-H // 16)), total // 128, 32)))
+                                                  max(1, min(ops.compute_units() // max(1, T * -(-H // 16)), total // 64, 64)), max_new_tokens=1)
             add(name, "paged_attention decode", launch, nbytes=float(reqs) * total * D * 2)
         else:
             tiles = -(-T // tq)

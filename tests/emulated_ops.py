@@ -236,8 +236,15 @@ LATENT_MAX_RANK = 1024
 ACTIVATIONS = {"none": 0, "relu2": 1}
 
 
-def latent_tile_tokens(heads):
-    return max(1, LATENT_ATTENTION_ROWS // min(heads, LATENT_ATTENTION_ROWS))
+LATENT_MFMA_ROWS = 64
+
+
+def latent_tile_tokens(heads, rows=LATENT_ATTENTION_ROWS):
+    return max(1, rows // min(heads, LATENT_ATTENTION_ROWS))
+
+
+def latent_attention_mfma_fits(dtype, heads, rank, rot):
+    return False
 
 
 def _turn(x, positions, inv_freq):
@@ -279,7 +286,7 @@ def rotate_pairs(src, src_head, src_off, dst, dst_head, dst_off, positions, inv_
 
 
 def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles, tile_tokens, heads, rank, rot,
-                     page_size, scale, sink, splits=1):
+                     page_size, scale, sink, splits=1, general=False, max_new_tokens=None):
     D = rank + rot
     for tile in range(num_tiles):
         if tile_req is None:
@@ -301,7 +308,7 @@ def latent_attention(q, out, plane, block_table, req_indptr, ctx_lens, tile_req,
             out[first + i] = ((e / den) @ rows[:, :rank]).reshape(-1).to(out.dtype)
 
 
-def heads_linear(x, x_head, weight, out, out_head):
+def heads_linear(x, x_head, weight, out, out_head, general=False):
     G, N, K = weight.shape
     for g in range(G):
         out[:, g * out_head: g * out_head + N] = (x[:, g * x_head: g * x_head + K].float() @ weight[g].float().T).to(out.dtype)
@@ -311,7 +318,7 @@ def _act(y, activation):
     return torch.clamp(y, min=0) ** 2 if activation == "relu2" else y
 
 
-def experts_linear(x, slot_token, weight, offsets, out, activation="none"):
+def experts_linear(x, slot_token, weight, offsets, out, activation="none", general=False):
     for e in range(weight.shape[0]):
         lo, hi = int(offsets[e]), int(offsets[e + 1])
         if hi > lo:

@@ -187,9 +187,11 @@ def _plain_latent_attention(q, rows_of, ctx_lens, new_lens, heads, rank, rot, sc
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tile_rows", [16, 64])
 @pytest.mark.parametrize("heads,rank,rot,page,splits,with_sink", [(6, 64, 32, 16, 1, True), (3, 40, 8, 4, 3, True), (20, 72, 16, 8, 2, False),
-                                                                   (1, 130, 0, 16, 1, True)])
-def test_latent_attention_against_formula(dtype, heads, rank, rot, page, splits, with_sink):
+                                                                   (1, 130, 0, 16, 1, True), (16, 128, 32, 16, 2, True), (5, 192, 64, 8, 1, False),
+                                                                   (2, 64, 0, 4, 3, True), (9, 512, 64, 16, 1, True)])
+def test_latent_attention_against_formula(dtype, heads, rank, rot, page, splits, with_sink, tile_rows):
     """Portions and single tokens in one call, over pages handed out in a scrambled order; one request's last query leans
     on its first key, far back, and its sink is large enough to show when it is left out."""
     from torchlet_amd.kernels import ops
@@ -217,7 +219,11 @@ def test_latent_attention_against_formula(dtype, heads, rank, rot, page, splits,
     q[37 + 1 + 8] = (rows_of[2][0] * 0.8).to(dtype)    # the last token of request 2 looks for its first key
     sink = (torch.randn(heads, generator=g) * 2 + 3) if with_sink else None
     scale = 0.3
-    tq = ops.latent_tile_tokens(heads)
+    on_matrix_cores = ops.latent_attention_mfma_fits(dtype, heads, rank, rot)
+    assert on_matrix_cores == (dtype == torch.bfloat16 and (rank + rot) % 32 == 0 and rank % 64 == 0)
+    if tile_rows > 16 and not on_matrix_cores:
+        pytest.skip("tiles of more than 16 rows are the matrix-core kernel's")
+    tq = ops.latent_tile_tokens(heads, tile_rows)
     tile_req, tile_tok0 = [], []
     for r, n in enumerate(new_lens):
         for t0 in range(0, n, tq):
@@ -226,23 +232,30 @@ def test_latent_attention_against_formula(dtype, heads, rank, rot, page, splits,
     out = torch.empty(T, heads * rank, dtype=dtype, device="cuda")
     ops.latent_attention(q.view(T, heads * D).cuda(), out, plane.cuda(), table.cuda(), indptr.cuda(), torch.tensor(ctx_lens, dtype=torch.int32).cuda(),
                          torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq,
-                         heads, rank, rot, page, scale, sink.cuda() if with_sink else None, splits)
+                         heads, rank, rot, page, scale, sink.cuda() if with_sink else None, splits, max_new_tokens=max(new_lens))
     want = _plain_latent_attention(q.double(), rows_of, ctx_lens, new_lens, heads, rank, rot, scale, sink.double() if with_sink else None)
     torch.testing.assert_close(out.cpu().double().view(T, heads, rank), want, **_tol(dtype))
+    if on_matrix_cores:        # the general kernel on the same operands
+        out2 = torch.empty_like(out)
+        if tile_rows == 16:
+            ops.latent_attention(q.view(T, heads * D).cuda(), out2, plane.cuda(), table.cuda(), indptr.cuda(), torch.tensor(ctx_lens, dtype=torch.int32).cuda(),
+                                 torch.tensor(tile_req, dtype=torch.int32).cuda(), torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq,
+                                 heads, rank, rot, page, scale, sink.cuda() if with_sink else None, splits, general=True)
+            torch.testing.assert_close(out2.cpu().double().view(T, heads, rank), want, **_tol(dtype))
     if with_sink:          # the sink matters here: left out, the result would be off by far more than the tolerance
         without = _plain_latent_attention(q.double(), rows_of, ctx_lens, new_lens, heads, rank, rot, scale, None)
         assert float((without - want).abs().max()) > 0.05
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_latent_attention_decode_without_tile_list(dtype):
+@pytest.mark.parametrize("heads,rank,rot,page", [(5, 48, 16, 8), (8, 64, 32, 8), (24, 256, 64, 16)])
+def test_latent_attention_decode_without_tile_list(dtype, heads, rank, rot, page):
     from torchlet_amd.kernels import ops
     g = torch.Generator().manual_seed(9)
-    heads, rank, rot, page = 5, 48, 16, 8
     D = rank + rot
     ctx_lens = [300, 0, 17]
     table = torch.zeros(3, 40, dtype=torch.int32)
-    plane = torch.full((60, 1, page, D), 1e4, dtype=dtype)
+    plane = torch.full((64, 1, page, D), 1e4, dtype=dtype)
     rows_of, nxt = [], 1
     for r, c in enumerate(ctx_lens):
         rows = torch.randn(c + 1, D, generator=g).to(dtype)
@@ -263,28 +276,29 @@ def test_latent_attention_decode_without_tile_list(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_heads_linear(dtype):
+@pytest.mark.parametrize("T,G,N,K,gap", [(70, 3, 37, 22, 6), (70, 3, 37, 64, 8), (1, 5, 300, 32, 0), (33, 2, 64, 96, 16), (16, 1, 130, 160, 8)])
+def test_heads_linear(dtype, T, G, N, K, gap):
+    """Sizes the matrix-core kernel takes (bfloat16, K a multiple of 32, aligned rows) and sizes it leaves to the general one."""
     from torchlet_amd.kernels import ops
     g = torch.Generator().manual_seed(11)
-    T, G, N, K = 70, 3, 37, 22
-    x = torch.randn(T, G * (K + 6) + 2, generator=g).to(dtype)
+    x = torch.randn(T, G * (K + gap) + (8 if K % 32 == 0 else 2), generator=g).to(dtype)
     w = torch.randn(G, N, K, generator=g).to(dtype)
     out = torch.zeros(T, G * (N + 3), dtype=dtype, device="cuda")
-    ops.heads_linear(x.cuda(), K + 6, w.cuda(), out, N + 3)
+    ops.heads_linear(x.cuda(), K + gap, w.cuda(), out, N + 3)
     got = out.cpu().double()
     for h in range(G):
-        want = x[:, h * (K + 6): h * (K + 6) + K].double() @ w[h].double().T
+        want = x[:, h * (K + gap): h * (K + gap) + K].double() @ w[h].double().T
         torch.testing.assert_close(got[:, h * (N + 3): h * (N + 3) + N], want, **_tol(dtype, 4))
         assert float(got[:, h * (N + 3) + N: (h + 1) * (N + 3)].abs().max()) == 0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,F", [(24, 19), (64, 96)])
 @pytest.mark.parametrize("T,experts,top", [(1, 4, 2), (150, 7, 3), (33, 5, 5), (64, 16, 1)])
-def test_routed_products(dtype, T, experts, top):
+def test_routed_products(dtype, T, experts, top, H, F):
     """The choice (ties go to the lower index), the weights, the sort by expert, and both products with the weighted sum."""
     from torchlet_amd.kernels import ops
     g = torch.Generator().manual_seed(T + experts)
-    H, F = 24, 19
     logits = torch.randn(T, experts, generator=g)
     logits[0, :] = 0.5                         # a tie over all experts: the lowest indices win
     weights, offsets, slot_token, pair_slot = ops.route(logits.cuda(), top)

@@ -88,13 +88,113 @@ grouped_gemm_kernel(const T* __restrict__ a, int a_ld, int a_group, const int* _
     }
 }
 
+// The same product on the matrix cores (bfloat16, K a multiple of 32, 16-byte aligned rows): both operands have K side by
+// side in memory, which is how v_mfma_f32_16x16x32_bf16 wants them, so a lane fetches its 16-byte pieces straight from
+// memory (the weights' once per tile of rows, the rows' from the caches) and nothing passes through shared memory.  The
+// weights are the first operand, so that a lane ends up with four neighbouring output columns of one row.  A work-group
+// of four waves owns a tile of 32 rows x 256 columns (one wave: 32 x 64); few rows per group (a decode step's experts)
+// leave half of each product empty, which costs nothing where the weights' stream sets the time.
+#define GM_BM 32
+#define GM_BN 256
+
+typedef __bf16 gm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gm_f32x4 __attribute__((ext_vector_type(4)));
+union GmFrag {
+    uint4 u;
+    gm_bf16x8 v;
+};
+
+__global__ void __launch_bounds__(256)
+grouped_gemm_mfma_kernel(const bf16_t* __restrict__ a, int a_ld, int a_group, const int* __restrict__ src, const bf16_t* __restrict__ w,
+                         bf16_t* __restrict__ out, int out_ld, int out_group, const int* __restrict__ offsets, int groups, int rows,
+                         int N, int K, int act) {
+    int g, m0, m_end;
+    if (offsets == nullptr) {
+        g = blockIdx.z; m0 = blockIdx.x * GM_BM; m_end = rows;
+        if (m0 >= m_end) return;
+    } else {
+        int tile = blockIdx.x;
+        g = 0; m0 = -1; m_end = 0;
+        for (int e = 0; e < groups; ++e) {
+            const int lo = offsets[e], hi = offsets[e + 1], tiles = (hi - lo + GM_BM - 1) / GM_BM;
+            if (tile < tiles) { g = e; m0 = lo + tile * GM_BM; m_end = hi; break; }
+            tile -= tiles;
+        }
+        if (m0 < 0) return;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.y * GM_BN + wave * 64;
+    if (n0 >= N) return;
+    const bf16_t* wg = w + (size_t)g * N * K;
+    const int a_col = offsets == nullptr ? g * a_group : 0, out_col = offsets == nullptr ? g * out_group : 0;
+    // this lane's rows of the two operands: weight row n0 + 16 i + li (clamped), x row of tile row 16 j + li (clamped)
+    const bf16_t* wrow[4];
+    const bf16_t* xrow[2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wrow[i] = wg + (size_t)min(n0 + 16 * i + li, N - 1) * K + 8 * kg;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int m = min(m0 + 16 * j + li, m_end - 1);
+        xrow[j] = a + (size_t)(src ? src[m] : m) * a_ld + a_col + 8 * kg;
+    }
+    const bool second = m0 + 16 < m_end;                // the tile has rows beyond its first 16
+    gm_f32x4 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = gm_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int k = 0; k < K; k += 32) {
+        GmFrag wf[4], xf[2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wf[i].u = *(const uint4*)(wrow[i] + k);
+        xf[0].u = *(const uint4*)(xrow[0] + k);
+        if (second) xf[1].u = *(const uint4*)(xrow[1] + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[i][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, xf[0].v, acc[i][0], 0, 0, 0);
+            if (second) acc[i][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, xf[1].v, acc[i][1], 0, 0, 0);
+        }
+    }
+    // acc[i][j][v] = out[row 16 j + li][column n0 + 16 i + 4 kg + v]
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int m = m0 + 16 * j + li;
+        if (m >= m_end) continue;
+        bf16_t* orow = out + (size_t)m * out_ld + out_col;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 16 * i + 4 * kg;
+            if (n + 3 < N && ((out_ld | out_col) & 3) == 0) {
+                union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(activate(acc[i][j][v], act)).bits;
+                *(uint2*)(orow + n) = pk.u;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N) orow[n + v] = from_float<bf16_t>(activate(acc[i][j][v], act));
+            }
+        }
+    }
+}
+
 extern "C" int tl_grouped_gemm(const void* a, int a_ld, int a_group, const void* src, const void* w, void* out, int out_ld, int out_group,
-                               const void* offsets, int groups, int rows, int N, int K, int act, int dtype, hipStream_t stream) {
+                               const void* offsets, int groups, int rows, int N, int K, int act, int dtype, int general, hipStream_t stream) {
     TL_REQUIRE(groups > 0 && rows >= 0 && N > 0 && K > 0 && a_ld > 0 && out_ld > 0, "grouped_gemm: bad sizes");
     TL_REQUIRE(act == ACT_NONE || act == ACT_RELU2, "grouped_gemm: unknown activation %d", act);
     if (rows == 0) return TL_OK;
     // with offsets, `rows` is the number of sorted slots in all groups together: every group may end in a partial tile
     dim3 grid(offsets ? (rows + GG_T - 1) / GG_T + groups : (rows + GG_T - 1) / GG_T, (N + GG_T - 1) / GG_T, offsets ? 1 : groups), block(256);
+    const bool aligned = K % 32 == 0 && a_ld % 8 == 0 && a_group % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0 &&
+                         ((uintptr_t)out % 8) == 0;
+    if (dtype == TL_DT_BF16 && aligned && !general) {
+        dim3 mgrid(offsets ? (rows + GM_BM - 1) / GM_BM + groups : (rows + GM_BM - 1) / GM_BM, (N + GM_BN - 1) / GM_BN, offsets ? 1 : groups);
+        grouped_gemm_mfma_kernel<<<mgrid, block, 0, stream>>>((const bf16_t*)a, a_ld, a_group, (const int*)src, (const bf16_t*)w, (bf16_t*)out, out_ld,
+                                                              out_group, (const int*)offsets, groups, rows, N, K, act);
+        TL_CHECK_LAUNCH("grouped_gemm_mfma");
+        return TL_OK;
+    }
     if (dtype == TL_DT_F32)
         grouped_gemm_kernel<float><<<grid, block, 0, stream>>>((const float*)a, a_ld, a_group, (const int*)src, (const float*)w, (float*)out, out_ld,
                                                                out_group, (const int*)offsets, groups, rows, N, K, act);

@@ -242,18 +242,279 @@ __global__ void latent_merge_kernel(const float* __restrict__ part_o, const floa
     }
 }
 
+// ------------------------------------------------------------------ attention on the matrix cores (bfloat16)
+// The same attention with both products on v_mfma_f32_16x16x32_bf16, transposed so that no result changes layout on its
+// way into the next product: S^T = K Q^T (a lane holds four keys of one query), O^T = L^T P^T (L the latent part of the
+// cached rows).  The first product sums over a row's numbers, which lie side by side in the cache; the second sums over
+// keys, so it wants the latents of neighbouring keys side by side: a step's 32 rows go to shared memory twice, as they
+// lie in the cache and transposed, written there once by the whole work-group.
+// A work-group of four waves owns RB blocks of 16 rows (row = token x head of a chunk of up to 16 heads; RB = 4, 2 or 1
+// by how many rows a tile of the step can have) and 4 / RB waves share a block: each takes all of the block's scores
+// (the softmax's state is then the same in all of them, nothing is exchanged) and its own share of the latent's columns.
+#define LM_KEYS 32                    // keys of a step
+#define LM_DC_MAX 20                  // 32-number pieces of a cache row (rows of up to 640 numbers)
+#define LM_LOG2E 1.4426950408889634f
+#define LM_BT_MAX 1536                // block-table entries of a request that a work-group keeps in shared memory (two work-groups fit a compute unit)
+
+typedef __bf16 lm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lm_f32x4 __attribute__((ext_vector_type(4)));
+union LmFrag {
+    uint4 u;
+    uint2 h[2];
+    lm_bf16x8 v;
+};
+
+template <int RB>
+__global__ void __launch_bounds__(256)
+latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __restrict__ out, const bf16_t* __restrict__ plane,
+                             const int* __restrict__ block_table, int bt_stride, const int* __restrict__ req_indptr,
+                             const int* __restrict__ ctx_lens, const int* __restrict__ tile_req, const int* __restrict__ tile_tok0,
+                             int tile_tokens, int heads, int rank, int rot, int page_size, float scale, const float* __restrict__ sink,
+                             int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    constexpr int WPR = 4 / RB;                      // waves that share a block of rows
+    constexpr int NT = 32 / WPR;                     // most blocks of 16 latent columns a wave sums (latents of up to 512 numbers)
+    extern __shared__ __align__(16) unsigned char lm_smem[];
+    const int D = rank + rot, dc = D / 32, ldk = D + 8, ldt = LM_KEYS + 4;
+    bf16_t* sk = (bf16_t*)lm_smem;                   // [32 keys][D + 8]: rows as they lie in the cache
+    bf16_t* st = sk + LM_KEYS * ldk;                 // [rank][32 + 4]: the latents transposed
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, g = lane >> 4;
+    const int rb = wave / WPR, share = wave % WPR;
+    const int tile = blockIdx.x, head0 = blockIdx.y * 16, split = blockIdx.z;
+    const int hchunk = min(16, heads - head0);
+    const int req = tile_req ? tile_req[tile] : tile, tok0 = tile_req ? tile_tok0[tile] : 0;
+    const int first = req_indptr ? req_indptr[req] : req, n_new = req_indptr ? req_indptr[req + 1] - first : 1;
+    const int ctx = ctx_lens[req];
+    const int ntok = min(tile_tokens, n_new - tok0);
+    const int rows = ntok * hchunk;
+    // the query this lane's column of S^T belongs to
+    const int row = rb * 16 + li;
+    const bool row_ok = row < rows;
+    const int rt = row_ok ? row / hchunk : 0, rh = head0 + (row_ok ? row % hchunk : 0);
+    const int tok = first + tok0 + rt, qpos = ctx + tok0 + rt;
+    LmFrag qf[LM_DC_MAX];
+#pragma unroll
+    for (int c = 0; c < LM_DC_MAX; ++c)
+        qf[c].u = (c < dc && row_ok) ? *(const uint4*)(q + (size_t)tok * q_ld + (size_t)rh * D + 32 * c + 8 * g) : make_uint4(0, 0, 0, 0);
+    const int nt = rank / 16 / WPR;                  // blocks of 16 latent columns of this wave: t0 .. t0 + nt - 1
+    const int t0 = share * nt;
+    lm_f32x4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = lm_f32x4{0.f, 0.f, 0.f, 0.f};
+    const bool with_sink = sink != nullptr && split == 0;
+    float m = with_sink ? sink[rh] * LM_LOG2E : -INFINITY;      // base 2: scores are taken times scale * log2(e)
+    float l = (with_sink && g == 0) ? 1.f : 0.f;                // (a lane sums its own keys; the lanes of a query are added at the end)
+    const float scale2 = scale * LM_LOG2E;
+    const int last = ctx + tok0 + ntok - 1;
+    const int* table = block_table + (size_t)req * bt_stride;
+    // A step's 32 rows come through registers: a wave brings 8 of them, lane (key = lane % 8, piece = lane / 8 + 8 i) a
+    // 16-byte piece per round i, so that the lanes that write the transposed copy lie side by side along the keys: two
+    // neighbouring lanes (an even key and the next) swap halves of their pieces and each writes four 32-bit words that hold
+    // both keys' numbers of one column.  The rows of the step after are requested before this step's products start and
+    // written when they are done.
+    const int pieces = D / 8, rounds = (pieces + 7) / 8;
+    const int kk = wave * 8 + (lane & 7), pg = lane >> 3;       // the key of the step that this lane brings, and its piece of a round
+    const bool odd = lane & 1;
+    // The request's block-table row lies in shared memory (the host sees to it that it fits): a step's rows are then one
+    // trip to memory, and, more to the point, looking a page up does not wait on the memory counter, which counts in order:
+    // a wait for a table entry would be a wait for every row requested before it, the rows of the steps ahead included.
+    int* tbl = (int*)(st + (size_t)rank * ldt);
+    for (int i = threadIdx.x; i <= last / page_size; i += 256) tbl[i] = table[i];
+    __syncthreads();
+    constexpr bool TWO = RB < 4;                     // steps requested ahead: two where the registers allow it
+    const int stride = splits * LM_KEYS, ahead = TWO ? 2 * stride : stride;
+    uint4 stage0[LM_DC_MAX / 2], stage1[TWO ? LM_DC_MAX / 2 : 1];
+    // (every lane fetches, from a clamped place where its own lies beyond the keys or the row: a fetch under a condition
+    // would be waited for on the spot; what must be zero is cleared when the pieces are written to shared memory)
+    auto request = [&](uint4 (&stage)[LM_DC_MAX / 2], int at) {
+        const int pos = min(at + kk, last);
+        const bf16_t* src = plane + ((size_t)tbl[pos / page_size] * page_size + pos % page_size) * D;
+#pragma unroll
+        for (int i = 0; i < LM_DC_MAX / 2; ++i)
+            if (i < rounds) stage[i] = *(const uint4*)(src + 8 * min(pg + 8 * i, pieces - 1));
+    };
+    auto step = [&](uint4 (&stage)[LM_DC_MAX / 2], int k0) {
+        __syncthreads();                             // the products of the step before have read shared memory
+#pragma unroll
+        for (int i = 0; i < LM_DC_MAX / 2; ++i) {
+            if (i < rounds) {
+                const int col = 64 * i + 8 * pg;
+                const uint4 x = (k0 + kk <= last && col < D) ? stage[i] : make_uint4(0, 0, 0, 0);
+                // the neighbour's half: the even lane keeps its first four numbers and gets the neighbour's, the odd lane the last four
+                const uint32_t mine0 = odd ? x.z : x.x, mine1 = odd ? x.w : x.y;
+                const uint32_t got0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)(odd ? x.x : x.z), 0xB1, 0xF, 0xF, true);
+                const uint32_t got1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)(odd ? x.y : x.w), 0xB1, 0xF, 0xF, true);
+                if (col < D) {
+                    *(uint4*)(sk + kk * ldk + col) = x;
+                    if (col < rank) {
+                        const uint32_t a0 = odd ? got0 : mine0, b0 = odd ? mine0 : got0;      // (even key, odd key)
+                        const uint32_t a1 = odd ? got1 : mine1, b1 = odd ? mine1 : got1;
+                        uint32_t* dst = (uint32_t*)(st + (col + (odd ? 4 : 0)) * ldt + (kk & ~1));
+                        dst[0] = (a0 & 0xffffu) | (b0 << 16);
+                        dst[ldt / 2] = (a0 >> 16) | (b0 & 0xffff0000u);
+                        dst[ldt] = (a1 & 0xffffu) | (b1 << 16);
+                        dst[3 * (ldt / 2)] = (a1 >> 16) | (b1 & 0xffff0000u);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (k0 + ahead <= last) request(stage, k0 + ahead);
+#pragma unroll
+        for (int j = 0; j < LM_KEYS / 32; ++j) {
+            const int kbase = k0 + 32 * j;
+            // ---- scores of 32 keys, as two halves of 16
+            float sc[8];
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                lm_f32x4 sacc = lm_f32x4{0.f, 0.f, 0.f, 0.f};
+                const bf16_t* krow = sk + (32 * j + 16 * hf + li) * ldk + 8 * g;
+#pragma unroll
+                for (int c = 0; c < LM_DC_MAX; ++c) {
+                    if (c < dc) {
+                        LmFrag kf;
+                        kf.u = *(const uint4*)(krow + 32 * c);
+                        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sacc, 0, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = kbase + 16 * hf + 4 * g + v;
+                    sc[4 * hf + v] = (row_ok && key <= qpos) ? sacc[v] * scale2 : -INFINITY;
+                }
+            }
+            float mloc = sc[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mloc = fmaxf(mloc, sc[i]);
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float m_new = fmaxf(m, mloc);
+            const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+            const bool moved = __any(m_new != m);    // the sums are rescaled only when some query's maximum moved
+            LmFrag pf;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = (sc[i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_new);
+                psum += p;
+                pf.v[i] = (__bf16)p;
+            }
+            l = l * alpha + psum;
+            m = m_new;
+            // ---- O^T += L^T P^T over this wave's share of the latent's columns
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if (t < nt) {
+                    const bf16_t* lrow = st + (16 * (t0 + t) + li) * ldt + 32 * j + 4 * g;
+                    LmFrag vf;
+                    vf.h[0] = *(const uint2*)lrow;
+                    vf.h[1] = *(const uint2*)(lrow + 16);
+                    if (moved) acc[t] *= alpha;
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    };
+    const int kfirst = split * LM_KEYS;
+    if (kfirst <= last) request(stage0, kfirst);
+    if constexpr (TWO) {
+        if (kfirst + stride <= last) request(stage1, kfirst + stride);
+        for (int k0 = kfirst; k0 <= last; k0 += 2 * stride) {
+            step(stage0, k0);
+            if (k0 + stride <= last) step(stage1, k0 + stride);
+        }
+    } else {
+        for (int k0 = kfirst; k0 <= last; k0 += stride) step(stage0, k0);
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    if (splits == 1) {
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        bf16_t* o = out + ((size_t)tok * heads + rh) * rank;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if (t < nt) {
+                union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[t][v] * inv).bits;
+                *(uint2*)(o + 16 * (t0 + t) + 4 * g) = pk.u;
+            }
+        }
+    } else {
+        const size_t prow = ((size_t)tok * heads + rh) * splits + split;
+        float* o = part_o + prow * rank;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            if (t < nt) *(lm_f32x4*)(o + 16 * (t0 + t) + 4 * g) = acc[t];
+        if (share == 0 && g == 0) { part_ml[prow * 2] = m / LM_LOG2E; part_ml[prow * 2 + 1] = l; }       // the merge works in base e
+    }
+}
+
+static size_t lm_smem_bytes(int rank, int rot) { return sizeof(bf16_t) * ((size_t)LM_KEYS * (rank + rot + 8) + (size_t)rank * (LM_KEYS + 4)) + sizeof(int) * LM_BT_MAX; }
+
+// Whether the matrix-core kernel is built for these sizes: rows of a multiple of 32 numbers up to 640, latents of a
+// multiple of 64 numbers up to 512, 16-byte aligned query rows.
+static bool lm_fits(int rank, int rot, int q_ld, const void* q, const void* plane, int bt_stride) {
+    const int D = rank + rot;
+    return bt_stride <= LM_BT_MAX && D % 32 == 0 && D <= 32 * LM_DC_MAX && rank % 64 == 0 && rank <= 512 && q_ld % 8 == 0 &&
+           ((uintptr_t)q % 16) == 0 && ((uintptr_t)plane % 16) == 0 && lm_smem_bytes(rank, rot) <= 160 * 1024;
+}
+
+template <int RB>
+static int launch_lm(const void* q, int q_ld, void* out, const void* plane, const void* block_table, int bt_stride, const void* req_indptr,
+                     const void* ctx_lens, const void* tile_req, const void* tile_tok0, int num_tiles, int tile_tokens, int heads, int rank,
+                     int rot, int page_size, float scale, const void* sink, int splits, void* part_o, void* part_ml, hipStream_t stream) {
+    static size_t allowed = 48 * 1024;               // (per instance of the template)
+    const size_t smem = lm_smem_bytes(rank, rot);
+    auto kernel = latent_attention_mfma_kernel<RB>;
+    if (smem > allowed) {
+        if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+            tl_set_error("latent_attention: cannot get %zu bytes of shared memory", smem); return TL_ERR_HIP;
+        }
+        allowed = smem;
+    }
+    dim3 grid(num_tiles, (heads + 15) / 16, splits), block(256);
+    kernel<<<grid, block, smem, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, (const bf16_t*)plane, (const int*)block_table, bt_stride,
+                                          (const int*)req_indptr, (const int*)ctx_lens, (const int*)tile_req, (const int*)tile_tok0, tile_tokens,
+                                          heads, rank, rot, page_size, scale, (const float*)sink, splits, (float*)part_o, (float*)part_ml);
+    TL_CHECK_LAUNCH("latent_attention_mfma");
+    return TL_OK;
+}
+
+extern "C" int tl_latent_attention_mfma_fits(int rank, int rot, int q_ld) {
+    const int D = rank + rot;
+    return (D % 32 == 0 && D <= 32 * LM_DC_MAX && rank % 64 == 0 && rank <= 512 && q_ld % 8 == 0 && lm_smem_bytes(rank, rot) <= 160 * 1024) ? 1 : 0;
+}
+
 // q [tokens, q_ld]: per head rank + rot numbers (head h at column h * (rank + rot)); out [tokens, heads * rank];
 // plane [pages, page_size, rank + rot]; sink float [heads] or null; tile_req null: tile i is the one token of request i.
 extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const void* plane, const void* block_table, int bt_stride,
                                    const void* req_indptr, const void* ctx_lens, const void* tile_req, const void* tile_tok0,
                                    int num_tiles, int tokens, int tile_tokens, int heads, int rank, int rot, int page_size, float scale,
-                                   const void* sink, int splits, void* part_o, void* part_ml, int dtype, hipStream_t stream) {
+                                   const void* sink, int splits, void* part_o, void* part_ml, int dtype, int general, int max_new_tokens,
+                                   hipStream_t stream) {
     TL_REQUIRE(num_tiles >= 0 && heads > 0 && rank > 0 && rot >= 0 && page_size > 0 && tile_tokens > 0, "latent_attention: bad sizes");
     TL_REQUIRE(rank <= 16 * TL_WAVE, "latent_attention: built for latents of up to %d numbers, got %d", 16 * TL_WAVE, rank);
-    TL_REQUIRE(tile_tokens * min(heads, LAT_ROWS) <= LAT_ROWS, "latent_attention: a tile of %d tokens and %d heads has more than %d rows", tile_tokens, heads, LAT_ROWS);
     TL_REQUIRE(splits >= 1 && (splits == 1 || (part_o != nullptr && part_ml != nullptr)), "latent_attention: parts need their scratch");
     TL_REQUIRE(q_ld >= heads * (rank + rot), "latent_attention: query rows are too short");
     if (num_tiles == 0) return TL_OK;
+    const int tile_rows = min(tile_tokens, max(1, max_new_tokens)) * min(heads, 16);       // most rows a tile of this step has
+    if (dtype == TL_DT_BF16 && !general && lm_fits(rank, rot, q_ld, q, plane, bt_stride)) {
+        TL_REQUIRE(tile_tokens * min(heads, 16) <= 64, "latent_attention: a tile of %d tokens and %d heads has more than 64 rows", tile_tokens, heads);
+        int rc;
+#define TL_LM(RB) rc = launch_lm<RB>(q, q_ld, out, plane, block_table, bt_stride, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles, tile_tokens, \
+                                     heads, rank, rot, page_size, scale, sink, splits, part_o, part_ml, stream)
+        if (tile_rows <= 16) TL_LM(1); else if (tile_rows <= 32) TL_LM(2); else TL_LM(4);
+#undef TL_LM
+        if (rc != TL_OK) return rc;
+        if (splits > 1) {
+            const int rows = tokens * heads;
+            latent_merge_kernel<bf16_t><<<rows, 128, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, rows, rank, splits);
+            TL_CHECK_LAUNCH("latent_merge");
+        }
+        return TL_OK;
+    }
+    TL_REQUIRE(tile_tokens * min(heads, LAT_ROWS) <= LAT_ROWS, "latent_attention: a tile of %d tokens and %d heads has more than %d rows", tile_tokens, heads, LAT_ROWS);
     const int D = rank + rot;
     const size_t smem = sizeof(float) * ((size_t)LAT_KT * (D + 1) + (size_t)LAT_ROWS * D + LAT_ROWS * LAT_KT);
     TL_REQUIRE(smem <= 160 * 1024, "latent_attention: %zu bytes of shared memory for rows of %d numbers", smem, D);

@@ -797,9 +797,19 @@ LATENT_ATTENTION_ROWS = 16       # rows (tokens x heads) a work-group of the lat
 LATENT_MAX_RANK = 1024
 
 
-def latent_tile_tokens(heads: int) -> int:
-    """New tokens of one request that share a tile of the latent attention."""
-    return max(1, LATENT_ATTENTION_ROWS // min(heads, LATENT_ATTENTION_ROWS))
+LATENT_MFMA_ROWS = 64            # rows of a tile of its matrix-core kernel
+
+
+def latent_tile_tokens(heads: int, rows: int = LATENT_ATTENTION_ROWS) -> int:
+    """New tokens of one request that share a tile of ``rows`` rows of the latent attention (a row: a token and one of
+    up to 16 heads)."""
+    return max(1, rows // min(heads, LATENT_ATTENTION_ROWS))
+
+
+def latent_attention_mfma_fits(dtype: torch.dtype, heads: int, rank: int, rot: int) -> bool:
+    """Whether :func:`latent_attention` runs these sizes on the matrix cores (bfloat16, cache rows of a multiple of 32 numbers up
+    to 640, latents of a multiple of 64 numbers up to 512); it then takes tiles of up to 64 rows, else of up to 16."""
+    return dtype == torch.bfloat16 and bool(_lib("latent").tl_latent_attention_mfma_fits(c_int(rank), c_int(rot), c_int(heads * (rank + rot))))
 
 
 def latent_prepare(down: torch.Tensor, q_rank: int, rank: int, rot: int, rot_dims: int, wq: torch.Tensor, wkv: torch.Tensor, eps: float,
@@ -849,12 +859,14 @@ def rotate_pairs(src: torch.Tensor, src_head: int, src_off: int, dst: torch.Tens
 def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, block_table: torch.Tensor, req_indptr: torch.Tensor | None,
                      ctx_lens: torch.Tensor, tile_req: torch.Tensor | None, tile_tok0: torch.Tensor | None, num_tiles: int,
                      tile_tokens: int, heads: int, rank: int, rot: int, page_size: int, scale: float, sink: torch.Tensor | None,
-                     splits: int = 1) -> None:
+                     splits: int = 1, general: bool = False, max_new_tokens: int | None = None) -> None:
     """Causal attention of the step's tokens over their requests' cached rows ``plane [pages, 1, page, rank + rot]``: ``q [T,
     heads * (rank + rot)]`` holds per head the query brought into the cache row's shape, a score is the dot product of the two
     times ``scale``, the softmax's denominator also holds ``exp(sink[head])`` (float32 ``[heads]``; ``None``: no sink), and ``out
     [T, heads * rank]`` receives the weighted sums of the rows' first ``rank`` numbers.  ``tile_req = tile_tok0 = None``: every
-    request brings one token.  ``splits``: work-groups that share a tile's keys (merged afterwards)."""
+    request brings one token.  ``splits``: work-groups that share a tile's keys (merged afterwards).  bfloat16 at sizes that
+    :func:`latent_attention_mfma_fits` runs on the matrix cores (``general=True`` forces the general kernel); ``max_new_tokens``:
+    the most tokens a request brings in this step (default: ``tile_tokens``), by which the matrix-core kernel sizes its work-groups."""
     T = q.shape[0]
     D = rank + rot
     if q.stride(1) != 1 or q.shape[1] < heads * D or out.shape != (T, heads * rank) or not out.is_contiguous() or out.dtype != q.dtype:
@@ -885,7 +897,8 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
     _check(lib, lib.tl_latent_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(plane), _ptr(block_table), c_int(block_table.stride(0)),
                                         _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T),
                                         c_int(tile_tokens), c_int(heads), c_int(rank), c_int(rot), c_int(page_size), c_float(scale),
-                                        _ptr(sink), c_int(splits), _ptr(part_o), _ptr(part_ml), c_int(_dt(q, "latent_attention")), _stream()))
+                                        _ptr(sink), c_int(splits), _ptr(part_o), _ptr(part_ml), c_int(_dt(q, "latent_attention")),
+                                        c_int(1 if general else 0), c_int(tile_tokens if max_new_tokens is None else max_new_tokens), _stream()))
 
 
 # ------------------------------------------------------------- products over groups, routing
@@ -893,9 +906,10 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
 ACTIVATIONS = {"none": 0, "relu2": 1}
 
 
-def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int) -> None:
+def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int, general: bool = False) -> None:
     """Per head ``h``: ``out[:, h * out_head : h * out_head + N] = x[:, h * x_head : h * x_head + K] @ weight[h].T`` with
-    ``weight [heads, N, K]``; ``x`` and ``out`` may be views with longer rows."""
+    ``weight [heads, N, K]``; ``x`` and ``out`` may be views with longer rows.  bfloat16 with K a multiple of 32 and 16-byte aligned
+    rows runs on the matrix cores (``general=True`` forces the general kernel)."""
     G, N, K = weight.shape
     T = x.shape[0]
     if x.dtype != weight.dtype or out.dtype != x.dtype or x.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != T or not weight.is_contiguous() \
@@ -904,11 +918,11 @@ def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.
     lib = _lib("experts")
     _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(x_head), c_void_p(0), _ptr(weight), _ptr(out), c_int(out.stride(0)),
                                     c_int(out_head), c_void_p(0), c_int(G), c_int(T), c_int(N), c_int(K), c_int(0),
-                                    c_int(_dt(x, "heads_linear")), _stream()))
+                                    c_int(_dt(x, "heads_linear")), c_int(1 if general else 0), _stream()))
 
 
 def experts_linear(x: torch.Tensor, slot_token: torch.Tensor | None, weight: torch.Tensor, offsets: torch.Tensor, out: torch.Tensor,
-                   activation: str = "none") -> None:
+                   activation: str = "none", general: bool = False) -> None:
     """``out[slot] = act(x[row(slot)] @ weight[e].T)`` for the slots ``offsets[e] .. offsets[e + 1] - 1`` of every expert ``e``;
     ``row(slot)`` is ``slot_token[slot]`` (a token routed to the expert) or, without it, the slot itself.  ``weight [experts, N, K]``,
     ``out [slots, N]``."""
@@ -922,7 +936,7 @@ def experts_linear(x: torch.Tensor, slot_token: torch.Tensor | None, weight: tor
     lib = _lib("experts")
     _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(0), _ptr(slot_token), _ptr(weight), _ptr(out), c_int(N), c_int(0),
                                     _ptr(offsets), c_int(G), c_int(S), c_int(N), c_int(K), c_int(ACTIVATIONS[activation]),
-                                    c_int(_dt(x, "experts_linear")), _stream()))
+                                    c_int(_dt(x, "experts_linear")), c_int(1 if general else 0), _stream()))
 
 
 def route(logits: torch.Tensor, top: int):

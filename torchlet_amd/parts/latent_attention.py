@@ -20,7 +20,7 @@ from ..config.base import ConfigError
 from ..kernels import ops
 from .base import KEEP_COMPUTE, KEEP_FLOAT32, KEEP_STORED, MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
 
-_MIN_KEYS_PER_SPLIT = 128
+_MIN_KEYS_PER_SPLIT = 64        # a step of the matrix-core kernel
 
 
 @MIXERS.register("latent_attention")
@@ -38,7 +38,9 @@ class LatentAttention(Mixer):
         self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
         if self.position is not None and not hasattr(self.position, "inv_freq"):
             raise ConfigError("latent attention folds a rotation in pairs into its kernels; its position encoding must offer inv_freq")
-        self.tile_tokens = ops.latent_tile_tokens(self.heads)
+        # tiles of 64 rows where the matrix-core kernel is built for these sizes, of 16 for the general kernel
+        on_matrix_cores = torch.device(device).type == "cuda" and ops.latent_attention_mfma_fits(dtype, self.heads, self.rank, self.rot)
+        self.tile_tokens = ops.latent_tile_tokens(self.heads, ops.LATENT_MFMA_ROWS if on_matrix_cores else ops.LATENT_ATTENTION_ROWS)
         self.compute_units = ops.compute_units()
         self.w_down = self.w_dq_norm = self.w_dkv_norm = self.w_uq = self.w_uk_t = self.w_uv = self.sink = self.w_o = None
 
@@ -79,9 +81,9 @@ class LatentAttention(Mixer):
         self.w_o = self._place(tensors["o"], KEEP_COMPUTE)
 
     def _splits(self, ctx, tiles: int) -> int:
-        """Work-groups that share a tile's keys: enough to give every compute unit one, no part under 128 keys."""
+        """Work-groups that share a tile's keys: enough to give every compute unit one, no part under 64 keys."""
         groups = max(1, tiles * -(-self.heads // ops.LATENT_ATTENTION_ROWS))
-        return max(1, min(self.compute_units // groups, ctx.max_total_len // _MIN_KEYS_PER_SPLIT, 32))
+        return max(1, min(self.compute_units // groups, ctx.max_total_len // _MIN_KEYS_PER_SPLIT, 64))
 
     def forward(self, h, ctx, cache):
         T, n = h.shape[0], self.heads
@@ -107,7 +109,8 @@ class LatentAttention(Mixer):
             tile_req = tile_tok0 = None
         mixed_latent = torch.empty((T, n * self.rank), dtype=self.dtype, device=dev)
         ops.latent_attention(qrow, mixed_latent, plane, table, ctx.req_indptr, ctx.ctx_lens, tile_req, tile_tok0, tiles, self.tile_tokens,
-                             n, self.rank, self.rot, cache.page_size, self.scale, self.sink, self._splits(ctx, tiles))
+                             n, self.rank, self.rot, cache.page_size, self.scale, self.sink, self._splits(ctx, tiles),
+                             max_new_tokens=ctx.max_new_tokens)
         values = torch.empty((T, n * self.vdim), dtype=self.dtype, device=dev)
         ops.heads_linear(mixed_latent, self.rank, self.w_uv, values, self.vdim)
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, n * self.vdim):
