@@ -5,6 +5,12 @@
 // the value up-projection follows outside.  Norms, angles, scores, weights and sums are float.
 #include "common.h"
 
+// A barrier that orders shared memory only: __syncthreads() also waits for every fetch from memory that is on its
+// way (its fence covers global memory), which would end a prefetch at the first barrier after it.
+__device__ __forceinline__ void shared_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // The pair (u, v) at entries (2i, 2i + 1) turned by position * inv_freq[i].
 __device__ __forceinline__ void turn_pair(float u, float v, float pos, float f, float& a, float& b) {
     float s, c;
@@ -323,17 +329,22 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
     constexpr bool TWO = RB < 4;                     // steps requested ahead: two where the registers allow it
     const int stride = splits * LM_KEYS, ahead = TWO ? 2 * stride : stride;
     uint4 stage0[LM_DC_MAX / 2], stage1[TWO ? LM_DC_MAX / 2 : 1];
+    // where this lane's pieces go in shared memory does not change from step to step
+    bf16_t* const sk_mine = sk + kk * ldk + 8 * pg;
+    uint32_t* const st_mine = (uint32_t*)(st + (8 * pg + (odd ? 4 : 0)) * ldt + (kk & ~1));
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
     // (every lane fetches, from a clamped place where its own lies beyond the keys or the row: a fetch under a condition
     // would be waited for on the spot; what must be zero is cleared when the pieces are written to shared memory)
     auto request = [&](uint4 (&stage)[LM_DC_MAX / 2], int at) {
         const int pos = min(at + kk, last);
-        const bf16_t* src = plane + ((size_t)tbl[pos / page_size] * page_size + pos % page_size) * D;
+        const int blk = page_shift >= 0 ? pos >> page_shift : pos / page_size;
+        const bf16_t* src = plane + ((size_t)tbl[blk] * page_size + (pos - blk * page_size)) * D;
 #pragma unroll
         for (int i = 0; i < LM_DC_MAX / 2; ++i)
             if (i < rounds) stage[i] = *(const uint4*)(src + 8 * min(pg + 8 * i, pieces - 1));
     };
     auto step = [&](uint4 (&stage)[LM_DC_MAX / 2], int k0) {
-        __syncthreads();                             // the products of the step before have read shared memory
+        shared_barrier();                             // the products of the step before have read shared memory
 #pragma unroll
         for (int i = 0; i < LM_DC_MAX / 2; ++i) {
             if (i < rounds) {
@@ -344,11 +355,11 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
                 const uint32_t got0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)(odd ? x.x : x.z), 0xB1, 0xF, 0xF, true);
                 const uint32_t got1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)(odd ? x.y : x.w), 0xB1, 0xF, 0xF, true);
                 if (col < D) {
-                    *(uint4*)(sk + kk * ldk + col) = x;
+                    *(uint4*)(sk_mine + 64 * i) = x;
                     if (col < rank) {
                         const uint32_t a0 = odd ? got0 : mine0, b0 = odd ? mine0 : got0;      // (even key, odd key)
                         const uint32_t a1 = odd ? got1 : mine1, b1 = odd ? mine1 : got1;
-                        uint32_t* dst = (uint32_t*)(st + (col + (odd ? 4 : 0)) * ldt + (kk & ~1));
+                        uint32_t* dst = st_mine + 32 * i * ldt;
                         dst[0] = (a0 & 0xffffu) | (b0 << 16);
                         dst[ldt / 2] = (a0 >> 16) | (b0 & 0xffff0000u);
                         dst[ldt] = (a1 & 0xffffu) | (b1 << 16);
@@ -357,29 +368,43 @@ latent_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __r
                 }
             }
         }
-        __syncthreads();
+        shared_barrier();
         if (k0 + ahead <= last) request(stage, k0 + ahead);
 #pragma unroll
         for (int j = 0; j < LM_KEYS / 32; ++j) {
             const int kbase = k0 + 32 * j;
             // ---- scores of 32 keys, as two halves of 16
             float sc[8];
+            {
+                // four chains of products (two halves of keys, the pieces of a row dealt to two sums each): a product that
+                // adds to the one before it waits for it
+                lm_f32x4 s00 = lm_f32x4{0.f, 0.f, 0.f, 0.f}, s01 = s00, s10 = s00, s11 = s00;
+                const bf16_t* krow0 = sk + (32 * j + li) * ldk + 8 * g;
+                const bf16_t* krow1 = krow0 + 16 * ldk;
 #pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
-                lm_f32x4 sacc = lm_f32x4{0.f, 0.f, 0.f, 0.f};
-                const bf16_t* krow = sk + (32 * j + 16 * hf + li) * ldk + 8 * g;
-#pragma unroll
-                for (int c = 0; c < LM_DC_MAX; ++c) {
+                for (int c = 0; c < LM_DC_MAX; c += 2) {
                     if (c < dc) {
-                        LmFrag kf;
-                        kf.u = *(const uint4*)(krow + 32 * c);
-                        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sacc, 0, 0, 0);
+                        LmFrag k0f, k1f;
+                        k0f.u = *(const uint4*)(krow0 + 32 * c);
+                        k1f.u = *(const uint4*)(krow1 + 32 * c);
+                        s00 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0f.v, qf[c].v, s00, 0, 0, 0);
+                        s10 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1f.v, qf[c].v, s10, 0, 0, 0);
+                    }
+                    if (c + 1 < dc) {
+                        LmFrag k0f, k1f;
+                        k0f.u = *(const uint4*)(krow0 + 32 * (c + 1));
+                        k1f.u = *(const uint4*)(krow1 + 32 * (c + 1));
+                        s01 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0f.v, qf[c + 1].v, s01, 0, 0, 0);
+                        s11 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1f.v, qf[c + 1].v, s11, 0, 0, 0);
                     }
                 }
+                s00 += s01;
+                s10 += s11;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int key = kbase + 16 * hf + 4 * g + v;
-                    sc[4 * hf + v] = (row_ok && key <= qpos) ? sacc[v] * scale2 : -INFINITY;
+                    const int key = kbase + 4 * g + v;
+                    sc[v] = (row_ok && key <= qpos) ? s00[v] * scale2 : -INFINITY;
+                    sc[4 + v] = (row_ok && key + 16 <= qpos) ? s10[v] * scale2 : -INFINITY;
                 }
             }
             float mloc = sc[0];

@@ -3,6 +3,12 @@
 // activation type; queries, keys and values come in the activation type as the projection left them.
 #include "common.h"
 
+// A barrier that orders shared memory only: __syncthreads() also waits for every fetch from memory that is on its
+// way (its fence covers global memory), which would end a prefetch at the first barrier after it.
+__device__ __forceinline__ void shared_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ------------------------------------------------------------------ gates
 __device__ __forceinline__ float soft_cap(float z, float cap) { return cap > 0.f ? cap * tanhf(z / cap) : z; }
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
@@ -11,72 +17,146 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 // Per request and head a state of dim x vdim numbers S, dim numbers n and a running maximum m:
 //   m' = max(f + m, i);  S' = exp(f + m - m') S + exp(i - m') k v^T;  n' likewise with k alone;
 //   o  = S'^T q / (max(|n' . q|, exp(-m')) + denom_eps),        q scaled by qscale.
-// A work-group owns the columns [64 * blockIdx.x, +64) of one request's and head's S: a lane owns one
-// column, a wave the RPT rows [wave * RPT, +RPT) of it, in registers for all tokens of the step.  Every
-// work-group of a head keeps n and m for itself (they are cheap); the one of the first columns stores them.
-// Tokens are taken TB at a time: their q, k, v and gates go to shared memory, every wave runs the TB updates
-// of its rows and leaves its part of each token's sums over the rows, and the parts are added in the order of
-// the waves, so a token's result does not depend on how the step was cut.
-#define MLSTM_TB 8
-#define MLSTM_COLS 64
+// n is one more column of S, the one whose "value" is 1 for every token: S'[:, n] = keep S[:, n] + take k, and n . q is
+// that column's output.  A work-group owns COLS - 1 columns of one request's and head's S and a copy of the n column
+// (so nothing is exchanged between work-groups; the first one stores n and m, and all of them read n and m from a
+// copy taken before the launch, since a work-group may start after the first one has finished).  A lane owns one column and RPT rows of
+// it, in registers for all tokens of the step: with COLS = 64 a wave holds RPT rows, with 32 or 16 it holds two or
+// four groups of RPT rows side by side, which makes more and smaller work-groups where a step has few requests.
+// Tokens are taken TB at a time: their q, k, v go to shared memory, one wave turns their gates into decays (the capped
+// gates and the exponentials side by side, the running maximum one token after the other, as it is defined), every
+// lane runs the TB updates of its rows and leaves its rows' share of each token's sums, and the shares are added in the
+// order of the rows.  A share is always that of RPT rows whatever COLS is, so a token's result does not depend on how
+// the step was cut or on what else is in it.
+#define MLSTM_TB 16
 
-template <typename T, int RPT>
+template <typename T, int RPT, int COLS>
 __global__ void __launch_bounds__(1024)
 mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
                   const float* __restrict__ gates,          // [tokens, 2 * heads]: raw input gates, raw forget gates
-                  float* __restrict__ state, size_t slot_stride, const int* __restrict__ slots,
+                  float* __restrict__ state, size_t slot_stride, const int* __restrict__ slots, const float* __restrict__ before,
                   const int* __restrict__ req_indptr, float* __restrict__ out, int heads, int dim, int vdim,
                   float cap, float qscale, float denom_eps) {
+    constexpr int RG = TL_WAVE / COLS;                 // groups of RPT rows a wave holds side by side
     extern __shared__ float smem[];
     const int waves = blockDim.x / TL_WAVE, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
+    const int shares = waves * RG;                     // ceil(dim / RPT)
     float* sq = smem;                                  // [TB][dim]
     float* sk = sq + MLSTM_TB * dim;                   // [TB][dim]
-    float* sv = sk + MLSTM_TB * dim;                   // [TB][64]
-    float* sg = sv + MLSTM_TB * MLSTM_COLS;            // [TB][2]: log input gate, log forget gate
-    float* sm = sg + MLSTM_TB * 2;                     // [TB]: the running maximum after each token
-    float* part = sm + MLSTM_TB;                       // [TB][waves][65]: a wave's share of o (64 columns) and of n.q
+    float* sv = sk + MLSTM_TB * dim;                   // [TB][COLS]: the values of the tile's columns, 1 for the n column
+    float* sd = sv + MLSTM_TB * COLS;                  // [TB][4]: keep, take, m after the token, (log input gate)
+    float* part = sd + MLSTM_TB * 4;                   // [TB][shares][COLS]
 
-    const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * MLSTM_COLS;
+    const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * (COLS - 1);
     const int tok0 = req_indptr[req], tok1 = req_indptr[req + 1];
     if (tok0 >= tok1) return;
-    const int col = col0 + lane;
-    const bool col_ok = col < vdim;
-    const int row0 = wave * RPT;
+    const int c = lane % COLS, share = wave * RG + lane / COLS;
+    const bool is_n = c == COLS - 1;
+    const int col = col0 + c;
+    const bool col_ok = !is_n && col < vdim;
+    const int row0 = share * RPT;
     float* st = state + (size_t)slots[req] * slot_stride + (size_t)head * ((size_t)dim * vdim + dim + 1);
     float* st_n = st + (size_t)dim * vdim;
+    const float* nm = before + ((size_t)req * heads + head) * (dim + 1);      // n and m as they were before the launch
 
     float S[RPT];
 #pragma unroll
-    for (int r = 0; r < RPT; ++r) S[r] = (col_ok && row0 + r < dim) ? st[(size_t)(row0 + r) * vdim + col] : 0.f;
-    const bool n_ok = lane < RPT && row0 + lane < dim;      // lane r of a wave keeps n of the wave's row r
-    float n = n_ok ? st_n[row0 + lane] : 0.f;
-    float m = st_n[dim];
+    for (int r = 0; r < RPT; ++r) {
+        const int row = row0 + r;
+        S[r] = row < dim ? (is_n ? nm[row] : (col_ok ? st[(size_t)row * vdim + col] : 0.f)) : 0.f;
+    }
+    float m = nm[dim];                                 // (kept by the first wave, which turns the gates into decays)
 
+    // A batch's q, k, v and raw gates are fetched into registers while the batch before is worked on (16-byte pieces of the
+    // q and k rows where they are aligned), and go to shared memory, widened, when its sums have been read.
+    constexpr int VEC = 16 / (int)sizeof(T);           // numbers of a 16-byte piece
+    constexpr int QK_PF = (MLSTM_TB * 2 * RPT * RG + VEC * TL_WAVE - 1) / (VEC * TL_WAVE);     // pieces a thread fetches at most
+    constexpr int V_PF = MLSTM_TB * COLS / TL_WAVE;    // values a thread fetches at most
+    const bool vec_ok = dim % VEC == 0 && ld % VEC == 0 && k_off % VEC == 0 && ((uintptr_t)qkv % 16) == 0;
+    const int dv = dim / VEC;
+    uint4 qk_stage[QK_PF];
+    T v_stage[V_PF];
+    float g_stage[2] = {0.f, 0.f};
+    auto fetch = [&](int base) {
+        const int nb = min(MLSTM_TB, tok1 - base);
+        if (vec_ok) {
+#pragma unroll
+            for (int j = 0; j < QK_PF; ++j) {
+                const int idx = min((int)threadIdx.x + j * (int)blockDim.x, nb * 2 * dv - 1);       // (clamped: every lane fetches)
+                const int t = idx / (2 * dv), rem = idx % (2 * dv);
+                qk_stage[j] = *(const uint4*)(qkv + (size_t)(base + t) * ld + head * dim + (rem >= dv ? k_off : 0) + (rem % dv) * VEC);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < V_PF; ++j) {
+            const int idx = min((int)threadIdx.x + j * (int)blockDim.x, nb * COLS - 1);
+            const int vc = min(col0 + idx % COLS, vdim - 1);
+            v_stage[j] = qkv[(size_t)(base + idx / COLS) * ld + v_off + head * vdim + vc];
+        }
+        if (wave == 0) {
+            const float* g = gates + (size_t)(base + min(lane, nb - 1)) * 2 * heads;
+            g_stage[0] = g[head];
+            g_stage[1] = g[heads + head];
+        }
+    };
+    fetch(tok0);
     for (int base = tok0; base < tok1; base += MLSTM_TB) {
         const int nb = min(MLSTM_TB, tok1 - base);
-        __syncthreads();                               // the sums of the tokens before have been read
-        for (int i = threadIdx.x; i < nb * dim; i += blockDim.x) {
-            const int t = i / dim, d = i % dim;
-            const T* row = qkv + (size_t)(base + t) * ld + head * dim;
-            sq[t * dim + d] = to_float(row[d]) * qscale;
-            sk[t * dim + d] = to_float(row[k_off + d]);
+        shared_barrier();                               // the sums of the tokens before have been read
+        if (vec_ok) {
+#pragma unroll
+            for (int j = 0; j < QK_PF; ++j) {
+                const int idx = threadIdx.x + j * blockDim.x;
+                if (idx < nb * 2 * dv) {
+                    const int t = idx / (2 * dv), rem = idx % (2 * dv);
+                    const bool is_k = rem >= dv;
+                    float* dst = (is_k ? sk : sq) + t * dim + (rem % dv) * VEC;
+                    const T* piece = (const T*)&qk_stage[j];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) dst[e] = is_k ? to_float(piece[e]) : to_float(piece[e]) * qscale;
+                }
+            }
+        } else {
+            for (int i = threadIdx.x; i < nb * dim; i += blockDim.x) {
+                const int t = i / dim, d = i % dim;
+                const T* row = qkv + (size_t)(base + t) * ld + head * dim;
+                sq[t * dim + d] = to_float(row[d]) * qscale;
+                sk[t * dim + d] = to_float(row[k_off + d]);
+            }
         }
-        for (int i = threadIdx.x; i < nb * MLSTM_COLS; i += blockDim.x) {
-            const int t = i / MLSTM_COLS, c = col0 + i % MLSTM_COLS;
-            sv[i] = c < vdim ? to_float(qkv[(size_t)(base + t) * ld + v_off + head * vdim + c]) : 0.f;
+#pragma unroll
+        for (int j = 0; j < V_PF; ++j) {
+            const int idx = threadIdx.x + j * blockDim.x;
+            if (idx < nb * COLS) {
+                const int cc = idx % COLS;
+                sv[idx] = cc == COLS - 1 ? 1.f : (col0 + cc < vdim ? to_float(v_stage[j]) : 0.f);
+            }
         }
-        if (threadIdx.x < nb) {
-            const float* g = gates + (size_t)(base + threadIdx.x) * 2 * heads;
-            sg[threadIdx.x * 2] = soft_cap(g[head], cap);
-            sg[threadIdx.x * 2 + 1] = log_sigmoid(soft_cap(g[heads + head], cap));
+        if (wave == 0) {
+            // the capped gates side by side, the running maximum token after token (every lane walks the same chain, the
+            // gates come from shared memory), then the decays side by side
+            const float gi = soft_cap(g_stage[0], cap), gf = log_sigmoid(soft_cap(g_stage[1], cap));
+            if (lane < nb) { sd[lane * 4 + 3] = gi; sd[lane * 4 + 2] = gf; }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            float m_before = m, m_mine = m;
+            for (int t = 0; t < nb; ++t) {
+                const float m_new = fmaxf(sd[t * 4 + 2] + m, sd[t * 4 + 3]);
+                if (lane == t) { m_before = m; m_mine = m_new; }
+                m = m_new;
+            }
+            __builtin_amdgcn_wave_barrier();           // (every lane has read the gates before the maxima take their place)
+            if (lane < nb) {
+                sd[lane * 4] = expf(gf + m_before - m_mine);
+                sd[lane * 4 + 1] = expf(gi - m_mine);
+                sd[lane * 4 + 2] = m_mine;
+            }
         }
-        __syncthreads();
+        if (base + MLSTM_TB < tok1) fetch(base + MLSTM_TB);
+        shared_barrier();
         for (int t = 0; t < nb; ++t) {
-            const float gi = sg[t * 2], gf = sg[t * 2 + 1];
-            const float m_new = fmaxf(gf + m, gi);
-            const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
-            m = m_new;
-            const float tv = take * sv[t * MLSTM_COLS + lane];
+            const float keep = sd[t * 4], tv = sd[t * 4 + 1] * sv[t * COLS + c];
             const float* kt = sk + t * dim + row0;
             const float* qt = sq + t * dim + row0;
             float o = 0.f;
@@ -87,85 +167,105 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
                     o = fmaf(S[r], qt[r], o);
                 }
             }
-            float nq = 0.f;
-            if (n_ok) {
-                n = fmaf(take, kt[lane], keep * n);
-                nq = n * qt[lane];
-            }
-            nq = wave_sum(nq);
-            float* p = part + ((size_t)t * waves + wave) * (MLSTM_COLS + 1);
-            p[lane] = o;
-            if (lane == 0) p[MLSTM_COLS] = nq;
-            if (threadIdx.x == 0) sm[t] = m;
+            part[((size_t)t * shares + share) * COLS + c] = o;
         }
-        __syncthreads();
+        shared_barrier();
         for (int t = wave; t < nb; t += waves) {
-            float osum = 0.f, nq = 0.f;
-            for (int w = 0; w < waves; ++w) {
-                const float* p = part + ((size_t)t * waves + w) * (MLSTM_COLS + 1);
-                osum += p[lane];
-                nq += p[MLSTM_COLS];
+            if (lane < COLS) {
+                float osum = 0.f, nq = 0.f;
+                for (int w = 0; w < shares; ++w) {
+                    const float* p = part + ((size_t)t * shares + w) * COLS;
+                    osum += p[lane];
+                    nq += p[COLS - 1];
+                }
+                if (lane < COLS - 1 && col0 + lane < vdim)
+                    out[((size_t)(base + t) * heads + head) * vdim + col0 + lane] = osum / (fmaxf(fabsf(nq), expf(-sd[t * 4 + 2])) + denom_eps);
             }
-            if (col_ok)
-                out[((size_t)(base + t) * heads + head) * vdim + col] = osum / (fmaxf(fabsf(nq), expf(-sm[t])) + denom_eps);
         }
     }
 #pragma unroll
-    for (int r = 0; r < RPT; ++r)
-        if (col_ok && row0 + r < dim) st[(size_t)(row0 + r) * vdim + col] = S[r];
-    if (blockIdx.x == 0) {
-        if (n_ok) st_n[row0 + lane] = n;
-        if (threadIdx.x == 0) st_n[dim] = m;
+    for (int r = 0; r < RPT; ++r) {
+        const int row = row0 + r;
+        if (row < dim) {
+            if (col_ok) st[(size_t)row * vdim + col] = S[r];
+            else if (is_n && blockIdx.x == 0) st_n[row] = S[r];
+        }
     }
+    if (blockIdx.x == 0 && threadIdx.x == 0) st_n[dim] = m;
 }
 
-template <typename T, int RPT>
+// n and m of the step's requests and heads, copied out of their slots: before[(req, head)] = [n (dim), m].
+__global__ void mlstm_before_kernel(const float* __restrict__ state, size_t slot_stride, const int* __restrict__ slots,
+                                    float* __restrict__ before, int heads, int dim, int vdim) {
+    const int req = blockIdx.x / heads, head = blockIdx.x % heads;
+    const float* src = state + (size_t)slots[req] * slot_stride + (size_t)head * ((size_t)dim * vdim + dim + 1) + (size_t)dim * vdim;
+    float* dst = before + (size_t)blockIdx.x * (dim + 1);
+    for (int i = threadIdx.x; i <= dim; i += blockDim.x) dst[i] = src[i];
+}
+
+template <typename T, int RPT, int COLS>
 static int launch_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, const void* gates, void* state, size_t slot_stride,
-                             const void* slots, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
+                             const void* slots, const void* before, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
                              float cap, float qscale, float denom_eps, hipStream_t stream) {
-    const int waves = (dim + RPT - 1) / RPT;
-    const size_t smem = sizeof(float) * ((size_t)2 * MLSTM_TB * dim + MLSTM_TB * MLSTM_COLS + 3 * MLSTM_TB +
-                                         (size_t)MLSTM_TB * waves * (MLSTM_COLS + 1));
+    constexpr int RG = TL_WAVE / COLS;
+    const int shares = (dim + RPT - 1) / RPT, waves = (shares + RG - 1) / RG;
+    const size_t smem = sizeof(float) * ((size_t)2 * MLSTM_TB * dim + MLSTM_TB * COLS + 4 * MLSTM_TB + (size_t)MLSTM_TB * waves * RG * COLS);
     TL_REQUIRE(smem <= 160 * 1024, "mlstm_scan: %zu bytes of shared memory for dim %d", smem, dim);
-    auto kernel = mlstm_scan_kernel<T, RPT>;
-    if (smem > 48 * 1024) {
+    auto kernel = mlstm_scan_kernel<T, RPT, COLS>;
+    static size_t allowed = 48 * 1024;               // (per instance of the template)
+    if (smem > allowed) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) { tl_set_error("mlstm_scan: cannot get %zu bytes of shared memory: %s", smem, hipGetErrorString(e)); return TL_ERR_HIP; }
+        allowed = smem;
     }
-    dim3 grid((vdim + MLSTM_COLS - 1) / MLSTM_COLS, heads, requests), block(waves * TL_WAVE);
+    dim3 grid((vdim + COLS - 2) / (COLS - 1), heads, requests), block(waves * TL_WAVE);
+    mlstm_before_kernel<<<requests * heads, 128, 0, stream>>>((const float*)state, slot_stride, (const int*)slots, (float*)before, heads, dim, vdim);
+    TL_CHECK_LAUNCH("mlstm_before");
     kernel<<<grid, block, smem, stream>>>((const T*)qkv, ld, k_off, v_off, (const float*)gates, (float*)state, slot_stride,
-                                           (const int*)slots, (const int*)req_indptr, (float*)out, heads, dim, vdim, cap, qscale, denom_eps);
+                                           (const int*)slots, (const float*)before, (const int*)req_indptr, (float*)out, heads, dim, vdim, cap, qscale, denom_eps);
     TL_CHECK_LAUNCH("mlstm_scan");
     return TL_OK;
 }
 
+static int tl_mlstm_units = 256;       // compute units the column tiles are dealt to
+extern "C" void tl_mlstm_set_compute_units(int units) { if (units > 0) tl_mlstm_units = units; }
+
 // qkv [tokens, ld]: queries at column 0 (heads * dim), keys at k_off, values at v_off (heads * vdim); gates float
 // [tokens, 2 * heads]; state float [slots, heads, dim * vdim + dim + 1] with slot_stride floats between slots;
-// out float [tokens, heads * vdim].  Requests whose req_indptr range is empty are left alone.
+// out float [tokens, heads * vdim]; before: scratch of requests * heads * (dim + 1) floats.  Requests whose req_indptr range
+// is empty are left alone.
 extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, const void* gates, void* state, long slot_stride,
-                             const void* slots, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
+                             const void* slots, const void* before, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
                              float cap, float qscale, float denom_eps, int dtype, hipStream_t stream) {
     TL_REQUIRE(requests >= 0 && heads > 0 && dim > 0 && vdim > 0 && ld > 0, "mlstm_scan: bad sizes");
     TL_REQUIRE(dim <= 1024, "mlstm_scan: built for up to 1024 query/key dimensions per head, got %d", dim);
     TL_REQUIRE(slot_stride >= (long)heads * ((long)dim * vdim + dim + 1), "mlstm_scan: the state rows are too short");
-    if (requests == 0) return TL_OK;
-    // rows a thread keeps: few for small heads (more waves at work), at most 16 waves to a work-group
-    const int rpt = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 256 ? 16 : dim <= 512 ? 32 : 64;
-#define TL_MLSTM(R)                                                                                                            \
-    return dtype == TL_DT_F32                                                                                                  \
-        ? launch_mlstm_scan<float, R>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, req_indptr, out,       \
-                                      requests, heads, dim, vdim, cap, qscale, denom_eps, stream)                             \
-        : launch_mlstm_scan<bf16_t, R>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, req_indptr, out,      \
-                                       requests, heads, dim, vdim, cap, qscale, denom_eps, stream)
     TL_REQUIRE(dtype == TL_DT_F32 || dtype == TL_DT_BF16, "mlstm_scan: unknown dtype %d", dtype);
+    if (requests == 0) return TL_OK;
+    // rows a lane keeps: few for small heads (more waves at work), at most 16 shares of them to a work-group of 64 columns
+    const int rpt = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 256 ? 16 : dim <= 512 ? 32 : 64;
+    // columns of a work-group: as few as it takes to give every compute unit one (the sums do not depend on the choice)
+    const long heads_reqs = (long)heads * requests;
+    const int cols = heads_reqs * ((vdim + 62) / 63) >= tl_mlstm_units ? 64 : heads_reqs * ((vdim + 30) / 31) >= tl_mlstm_units ? 32 : 16;
+#define TL_MLSTM_C(R, C)                                                                                                       \
+    return dtype == TL_DT_F32                                                                                                  \
+        ? launch_mlstm_scan<float, R, C>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, before, req_indptr, out,    \
+                                         requests, heads, dim, vdim, cap, qscale, denom_eps, stream)                          \
+        : launch_mlstm_scan<bf16_t, R, C>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, before, req_indptr, out,   \
+                                          requests, heads, dim, vdim, cap, qscale, denom_eps, stream)
+#define TL_MLSTM(R)                                  \
+    if (cols == 64) { TL_MLSTM_C(R, 64); }           \
+    else if (cols == 32) { TL_MLSTM_C(R, 32); }      \
+    else { TL_MLSTM_C(R, 16); }
     switch (rpt) {
-        case 4: TL_MLSTM(4);
-        case 8: TL_MLSTM(8);
-        case 16: TL_MLSTM(16);
-        case 32: TL_MLSTM(32);
-        default: TL_MLSTM(64);
+        case 4: TL_MLSTM(4)
+        case 8: TL_MLSTM(8)
+        case 16: TL_MLSTM(16)
+        case 32: TL_MLSTM(32)
+        default: TL_MLSTM(64)
     }
 #undef TL_MLSTM
+#undef TL_MLSTM_C
 }
 
 // ------------------------------------------------------------------ gated per-head norm

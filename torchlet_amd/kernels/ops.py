@@ -41,6 +41,8 @@ def _lib(name: str) -> ctypes.CDLL:
         _libs[name] = lib
         if name == "gemm" and torch.cuda.is_available():
             lib.tl_gemm_set_compute_units(c_int(compute_units()))
+        if name == "recurrent" and torch.cuda.is_available():
+            lib.tl_mlstm_set_compute_units(c_int(compute_units()))
     return lib
 
 
@@ -771,8 +773,9 @@ def mlstm_scan(qkv: torch.Tensor, k_off: int, v_off: int, gates: torch.Tensor, s
     _i32(slots, "slots", R)
     _i32(req_indptr, "req_indptr", R + 1)
     lib = _lib("recurrent")
+    before = torch.empty((R, heads, dim + 1), dtype=torch.float32, device=qkv.device)      # n and m as the step finds them
     _check(lib, lib.tl_mlstm_scan(_ptr(qkv), c_int(qkv.stride(0)), c_int(k_off), c_int(v_off), _ptr(gates), _ptr(state),
-                                  ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(req_indptr), _ptr(out), c_int(R), c_int(heads),
+                                  ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(before), _ptr(req_indptr), _ptr(out), c_int(R), c_int(heads),
                                   c_int(dim), c_int(vdim), c_float(cap if cap else 0.0), c_float(qscale), c_float(denom_eps),
                                   c_int(_dt(qkv, "mlstm_scan")), _stream()))
 

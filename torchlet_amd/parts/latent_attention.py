@@ -20,7 +20,7 @@ from ..config.base import ConfigError
 from ..kernels import ops
 from .base import KEEP_COMPUTE, KEEP_FLOAT32, KEEP_STORED, MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
 
-_MIN_KEYS_PER_SPLIT = 64        # a step of the matrix-core kernel
+_MIN_KEYS_PER_SPLIT = 64        # two steps of the matrix-core kernel
 
 
 @MIXERS.register("latent_attention")
