@@ -489,7 +489,7 @@ def migurax_sizes(size: str) -> tuple[dict, dict]:
     Qwen2 configuration of the same width, layer count, vocabulary and dense feed-forward width."""
     width, heads, ff, experts, eff, top, q_rank, mheads = dict(s=(2048, 16, 8192, 16, 1024, 2, 768, 4), m=(4096, 32, 16384, 32, 2048, 4, 1536, 8))[size]
     moe = dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, top=top))
-    rec = dict(heads=mheads, dim=256, vdim=512, gate_cap=15.0)
+    rec = dict(heads=mheads, dim=256, vdim=512, gate_cap=12.0)
     layers = [dict(type="mlstm", mixer=rec, mlp=dict(kind="dense", ff=ff)), _latent_layer(heads, 128, 64, 128, 512, q_rank, moe),
               _latent_layer(heads, 128, 64, 128, 512, q_rank, moe), dict(type="mlstm", mixer=rec, mlp=moe)]
     ours = dict(architecture="Migurax", vocab=32000, width=width, postln_alpha=1.0, norm=dict(eps=1e-5), layers=layers, max_positions=8192)
@@ -591,7 +591,7 @@ def migurax_kernels(ours: dict, like: dict, batch: int, context: int, tokens: in
         out = torch.empty(T, h * v, device=dev)
         slots = torch.arange(reqs, dtype=torch.int32, device=dev)
         indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
-        launch = lambda: ops.mlstm_scan(qkv, h * d, 2 * h * d, gates, state, slots, indptr, out, h, d, v, 15.0, d ** -0.5, 1e-6)
+        launch = lambda: ops.mlstm_scan(qkv, h * d, 2 * h * d, gates, state, slots, indptr, out, h, d, v, 12.0, d ** -0.5, 1e-6)
         if reqs > 1:
             add(name, "paged_attention decode", launch, nbytes=2.0 * reqs * h * d * v * 4)
         else:

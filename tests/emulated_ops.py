@@ -237,6 +237,7 @@ ACTIVATIONS = {"none": 0, "relu2": 1}
 
 
 LATENT_MFMA_ROWS = 64
+LATENT_MFMA_MAX_BLOCKS = 1536
 
 
 def latent_tile_tokens(heads, rows=LATENT_ATTENTION_ROWS):

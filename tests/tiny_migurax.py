@@ -26,7 +26,7 @@ CONFIGS = {
         dict(type="latent_attention", mixer=_latent(1, 16, 8, 8, 16, 32, 0.2, 5000.0, dims=4), mlp=_moe(24, 3, 1)),
     ]),
     "Q": dict(architecture="Migurax", vocab=131, width=72, postln_alpha=1.0, norm=dict(eps=3e-6), layers=[
-        dict(type="mlstm", mixer=dict(heads=4, dim=70, vdim=130, gate_cap=15.0), mlp=_moe(24, 4, 4)),
+        dict(type="mlstm", mixer=dict(heads=4, dim=70, vdim=130, gate_cap=14.0), mlp=_moe(24, 4, 4)),
         dict(type="latent_attention", mixer=_latent(20, 16, 8, 16, 32, 40, 0.25, 20000.0), mlp=dict(kind="dense", ff=96)),
     ]),
     "R": dict(architecture="Migurax", vocab=64, width=64, postln_alpha=3.0, norm=dict(eps=1e-6), layers=[

@@ -230,20 +230,35 @@ latent_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, 
 }
 
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row, in the order of the parts.
+// The parts' weights are worked out once per row (by the first threads, into shared memory), then every thread sums its
+// columns, neighbours reading neighbouring numbers.
+#define LAT_MAX_SPLITS 64
 template <typename T>
 __global__ void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ out,
                                     int rows, int rank, int splits) {
+    __shared__ float wgt[LAT_MAX_SPLITS];
+    __shared__ float inv_s;
     const int row = blockIdx.x;
     const float* ml = part_ml + (size_t)row * splits * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, ml[s * 2]);
-    float den = 0.f;
-    for (int s = 0; s < splits; ++s) den += (ml[s * 2] == -INFINITY) ? 0.f : expf(ml[s * 2] - M) * ml[s * 2 + 1];
-    const float inv = den > 0.f ? 1.f / den : 0.f;
+    if (threadIdx.x < TL_WAVE) {
+        const int s = threadIdx.x;
+        const float ms = s < splits ? ml[s * 2] : -INFINITY;
+        const float M = wave_max(ms);
+        const float w = (s < splits && ms != -INFINITY) ? expf(ms - M) : 0.f;
+        if (s < splits) wgt[s] = w;
+        float den = 0.f;
+        for (int i = 0; i < splits; ++i) {             // in the order of the parts
+            const float wi = __shfl(w, i, TL_WAVE), li = ml[i * 2 + 1];
+            den += wi * li;
+        }
+        if (s == 0) inv_s = den > 0.f ? 1.f / den : 0.f;
+    }
+    __syncthreads();
+    const float inv = inv_s;
+    const float* po = part_o + (size_t)row * splits * rank;
     for (int c = threadIdx.x; c < rank; c += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < splits; ++s)
-            if (ml[s * 2] != -INFINITY) a = fmaf(expf(ml[s * 2] - M), part_o[((size_t)row * splits + s) * rank + c], a);
+        for (int s = 0; s < splits; ++s) a = fmaf(wgt[s], po[(size_t)s * rank + c], a);
         out[(size_t)row * rank + c] = from_float<T>(a * inv);
     }
 }
@@ -520,7 +535,7 @@ extern "C" int tl_latent_attention(const void* q, int q_ld, void* out, const voi
                                    hipStream_t stream) {
     TL_REQUIRE(num_tiles >= 0 && heads > 0 && rank > 0 && rot >= 0 && page_size > 0 && tile_tokens > 0, "latent_attention: bad sizes");
     TL_REQUIRE(rank <= 16 * TL_WAVE, "latent_attention: built for latents of up to %d numbers, got %d", 16 * TL_WAVE, rank);
-    TL_REQUIRE(splits >= 1 && (splits == 1 || (part_o != nullptr && part_ml != nullptr)), "latent_attention: parts need their scratch");
+    TL_REQUIRE(splits >= 1 && splits <= LAT_MAX_SPLITS && (splits == 1 || (part_o != nullptr && part_ml != nullptr)), "latent_attention: 1 to 64 parts, with their scratch");
     TL_REQUIRE(q_ld >= heads * (rank + rot), "latent_attention: query rows are too short");
     if (num_tiles == 0) return TL_OK;
     const int tile_rows = min(tile_tokens, max(1, max_new_tokens)) * min(heads, 16);       // most rows a tile of this step has

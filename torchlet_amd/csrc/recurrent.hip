@@ -36,16 +36,18 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
                   const float* __restrict__ gates,          // [tokens, 2 * heads]: raw input gates, raw forget gates
                   float* __restrict__ state, size_t slot_stride, const int* __restrict__ slots, const float* __restrict__ before,
                   const int* __restrict__ req_indptr, float* __restrict__ out, int heads, int dim, int vdim,
-                  float cap, float qscale, float denom_eps) {
+                  float cap, float qscale, float denom_eps, int tb) {
     constexpr int RG = TL_WAVE / COLS;                 // groups of RPT rows a wave holds side by side
     extern __shared__ float smem[];
     const int waves = blockDim.x / TL_WAVE, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     const int shares = waves * RG;                     // ceil(dim / RPT)
-    float* sq = smem;                                  // [TB][dim]
-    float* sk = sq + MLSTM_TB * dim;                   // [TB][dim]
-    float* sv = sk + MLSTM_TB * dim;                   // [TB][COLS]: the values of the tile's columns, 1 for the n column
-    float* sd = sv + MLSTM_TB * COLS;                  // [TB][4]: keep, take, m after the token, (log input gate)
-    float* part = sd + MLSTM_TB * 4;                   // [TB][shares][COLS]
+    // tb <= MLSTM_TB tokens are taken at a time: no more than the longest request of the step brings, so that a decode step's
+    // work-groups need little shared memory and several fit a compute unit
+    float* sq = smem;                                  // [tb][dim]
+    float* sk = sq + tb * dim;                         // [tb][dim]
+    float* sv = sk + tb * dim;                         // [tb][COLS]: the values of the tile's columns, 1 for the n column
+    float* sd = sv + tb * COLS;                        // [tb][4]: keep, take, m after the token, (log input gate)
+    float* part = sd + tb * 4;                         // [tb][shares][COLS]
 
     const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * (COLS - 1);
     const int tok0 = req_indptr[req], tok1 = req_indptr[req + 1];
@@ -78,7 +80,7 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
     T v_stage[V_PF];
     float g_stage[2] = {0.f, 0.f};
     auto fetch = [&](int base) {
-        const int nb = min(MLSTM_TB, tok1 - base);
+        const int nb = min(tb, tok1 - base);
         if (vec_ok) {
 #pragma unroll
             for (int j = 0; j < QK_PF; ++j) {
@@ -100,8 +102,8 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
         }
     };
     fetch(tok0);
-    for (int base = tok0; base < tok1; base += MLSTM_TB) {
-        const int nb = min(MLSTM_TB, tok1 - base);
+    for (int base = tok0; base < tok1; base += tb) {
+        const int nb = min(tb, tok1 - base);
         shared_barrier();                               // the sums of the tokens before have been read
         if (vec_ok) {
 #pragma unroll
@@ -153,7 +155,7 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
                 sd[lane * 4 + 2] = m_mine;
             }
         }
-        if (base + MLSTM_TB < tok1) fetch(base + MLSTM_TB);
+        if (base + tb < tok1) fetch(base + tb);
         shared_barrier();
         for (int t = 0; t < nb; ++t) {
             const float keep = sd[t * 4], tv = sd[t * 4 + 1] * sv[t * COLS + c];
@@ -206,10 +208,10 @@ __global__ void mlstm_before_kernel(const float* __restrict__ state, size_t slot
 template <typename T, int RPT, int COLS>
 static int launch_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, const void* gates, void* state, size_t slot_stride,
                              const void* slots, const void* before, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
-                             float cap, float qscale, float denom_eps, hipStream_t stream) {
+                             float cap, float qscale, float denom_eps, int tb, hipStream_t stream) {
     constexpr int RG = TL_WAVE / COLS;
     const int shares = (dim + RPT - 1) / RPT, waves = (shares + RG - 1) / RG;
-    const size_t smem = sizeof(float) * ((size_t)2 * MLSTM_TB * dim + MLSTM_TB * COLS + 4 * MLSTM_TB + (size_t)MLSTM_TB * waves * RG * COLS);
+    const size_t smem = sizeof(float) * ((size_t)2 * tb * dim + tb * COLS + 4 * tb + (size_t)tb * waves * RG * COLS);
     TL_REQUIRE(smem <= 160 * 1024, "mlstm_scan: %zu bytes of shared memory for dim %d", smem, dim);
     auto kernel = mlstm_scan_kernel<T, RPT, COLS>;
     static size_t allowed = 48 * 1024;               // (per instance of the template)
@@ -222,7 +224,7 @@ static int launch_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
     mlstm_before_kernel<<<requests * heads, 128, 0, stream>>>((const float*)state, slot_stride, (const int*)slots, (float*)before, heads, dim, vdim);
     TL_CHECK_LAUNCH("mlstm_before");
     kernel<<<grid, block, smem, stream>>>((const T*)qkv, ld, k_off, v_off, (const float*)gates, (float*)state, slot_stride,
-                                           (const int*)slots, (const float*)before, (const int*)req_indptr, (float*)out, heads, dim, vdim, cap, qscale, denom_eps);
+                                           (const int*)slots, (const float*)before, (const int*)req_indptr, (float*)out, heads, dim, vdim, cap, qscale, denom_eps, tb);
     TL_CHECK_LAUNCH("mlstm_scan");
     return TL_OK;
 }
@@ -236,8 +238,9 @@ extern "C" void tl_mlstm_set_compute_units(int units) { if (units > 0) tl_mlstm_
 // is empty are left alone.
 extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, const void* gates, void* state, long slot_stride,
                              const void* slots, const void* before, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
-                             float cap, float qscale, float denom_eps, int dtype, hipStream_t stream) {
+                             float cap, float qscale, float denom_eps, int longest, int dtype, hipStream_t stream) {
     TL_REQUIRE(requests >= 0 && heads > 0 && dim > 0 && vdim > 0 && ld > 0, "mlstm_scan: bad sizes");
+    const int tb = longest < 1 ? 1 : (longest < MLSTM_TB ? longest : MLSTM_TB);       // longest: the most tokens a request of the step brings
     TL_REQUIRE(dim <= 1024, "mlstm_scan: built for up to 1024 query/key dimensions per head, got %d", dim);
     TL_REQUIRE(slot_stride >= (long)heads * ((long)dim * vdim + dim + 1), "mlstm_scan: the state rows are too short");
     TL_REQUIRE(dtype == TL_DT_F32 || dtype == TL_DT_BF16, "mlstm_scan: unknown dtype %d", dtype);
@@ -250,9 +253,9 @@ extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
 #define TL_MLSTM_C(R, C)                                                                                                       \
     return dtype == TL_DT_F32                                                                                                  \
         ? launch_mlstm_scan<float, R, C>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, before, req_indptr, out,    \
-                                         requests, heads, dim, vdim, cap, qscale, denom_eps, stream)                          \
+                                         requests, heads, dim, vdim, cap, qscale, denom_eps, tb, stream)                      \
         : launch_mlstm_scan<bf16_t, R, C>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, before, req_indptr, out,   \
-                                          requests, heads, dim, vdim, cap, qscale, denom_eps, stream)
+                                          requests, heads, dim, vdim, cap, qscale, denom_eps, tb, stream)
 #define TL_MLSTM(R)                                  \
     if (cols == 64) { TL_MLSTM_C(R, 64); }           \
     else if (cols == 32) { TL_MLSTM_C(R, 32); }      \

@@ -777,7 +777,7 @@ def mlstm_scan(qkv: torch.Tensor, k_off: int, v_off: int, gates: torch.Tensor, s
     _check(lib, lib.tl_mlstm_scan(_ptr(qkv), c_int(qkv.stride(0)), c_int(k_off), c_int(v_off), _ptr(gates), _ptr(state),
                                   ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(before), _ptr(req_indptr), _ptr(out), c_int(R), c_int(heads),
                                   c_int(dim), c_int(vdim), c_float(cap if cap else 0.0), c_float(qscale), c_float(denom_eps),
-                                  c_int(_dt(qkv, "mlstm_scan")), _stream()))
+                                  c_int(max(1, T - R + 1)), c_int(_dt(qkv, "mlstm_scan")), _stream()))
 
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, heads: int, vdim: int) -> None:
@@ -801,6 +801,7 @@ LATENT_MAX_RANK = 1024
 
 
 LATENT_MFMA_ROWS = 64            # rows of a tile of its matrix-core kernel
+LATENT_MFMA_MAX_BLOCKS = 1536    # block-table entries of a request that its work-groups keep in shared memory
 
 
 def latent_tile_tokens(heads: int, rows: int = LATENT_ATTENTION_ROWS) -> int:

@@ -41,6 +41,7 @@ class LatentAttention(Mixer):
         # tiles of 64 rows where the matrix-core kernel is built for these sizes, of 16 for the general kernel
         on_matrix_cores = torch.device(device).type == "cuda" and ops.latent_attention_mfma_fits(dtype, self.heads, self.rank, self.rot)
         self.tile_tokens = ops.latent_tile_tokens(self.heads, ops.LATENT_MFMA_ROWS if on_matrix_cores else ops.LATENT_ATTENTION_ROWS)
+        self.general_tile_tokens = ops.latent_tile_tokens(self.heads, ops.LATENT_ATTENTION_ROWS)
         self.compute_units = ops.compute_units()
         self.w_down = self.w_dq_norm = self.w_dkv_norm = self.w_uq = self.w_uk_t = self.w_uv = self.sink = self.w_o = None
 
@@ -104,13 +105,16 @@ class LatentAttention(Mixer):
         qrow = torch.empty((T, n * self.row), dtype=self.dtype, device=dev)
         ops.heads_linear(q, self.dim + self.rot, self.w_uk_t, qrow, self.row)
         ops.rotate_pairs(q, self.dim + self.rot, self.dim, qrow, self.row, self.rank, ctx.positions, inv_freq, n, self.rot)
-        tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
+        # (sequences whose block table the matrix-core kernel cannot keep in shared memory go to the general kernel and its tiles)
+        general = table.shape[1] > ops.LATENT_MFMA_MAX_BLOCKS
+        tq = self.general_tile_tokens if general else self.tile_tokens
+        tile_req, tile_tok0, tiles = ctx.tiles(tq)
         if ctx.decode_only and tiles == T:          # one token per request: no tile list to look up
             tile_req = tile_tok0 = None
         mixed_latent = torch.empty((T, n * self.rank), dtype=self.dtype, device=dev)
-        ops.latent_attention(qrow, mixed_latent, plane, table, ctx.req_indptr, ctx.ctx_lens, tile_req, tile_tok0, tiles, self.tile_tokens,
+        ops.latent_attention(qrow, mixed_latent, plane, table, ctx.req_indptr, ctx.ctx_lens, tile_req, tile_tok0, tiles, tq,
                              n, self.rank, self.rot, cache.page_size, self.scale, self.sink, self._splits(ctx, tiles),
-                             max_new_tokens=ctx.max_new_tokens)
+                             general=general, max_new_tokens=ctx.max_new_tokens)
         values = torch.empty((T, n * self.vdim), dtype=self.dtype, device=dev)
         ops.heads_linear(mixed_latent, self.rank, self.w_uv, values, self.vdim)
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, n * self.vdim):
