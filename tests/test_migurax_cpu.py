@@ -71,10 +71,10 @@ def test_cache_plan_has_a_state_per_recurrent_layer_and_one_page_group_per_row_s
     assert torch.equal(states[1][slot], fresh.caches[1].state[fresh.cache.slot("b")])
 
 
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "T"])
 @pytest.mark.parametrize("mode", ["whole", "tail_singles", "portions", "mixed"])
 def test_step_function_equals_plain_under_every_split(cpu_ops, folders, name, mode):
-    lengths = [37, 5, 70, 1, 18, 33] if name != "Q" else [21, 1, 30]
+    lengths = [37, 5, 70, 1, 18, 33] if name not in "QT" else [21, 1, 30]
     seqs, refs = tiny_migurax.clear_sequences(name, _weights(name), lengths)
     steps = scenarios.number(getattr(scenarios, mode)(seqs) if mode != "tail_singles" else scenarios.tail_singles(seqs, tail=9))
     page = tiny_migurax.PAGE_SIZES[name]

@@ -60,12 +60,12 @@ def _replay(runner, steps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "T"])
 def test_every_way_of_cutting_requests_equals_plain(folders, name, dtype):
     """Whole requests; most of a request and its last tokens one by one; portions of changing size down to two tokens; up to
     four live requests with portions beside single tokens, in a pool that holds no more than the live ones need, so pages and
     slots are used again."""
-    lengths = [37, 5, 70, 1, 18, 33] if name != "Q" else [21, 1, 30]
+    lengths = [37, 5, 70, 1, 18, 33] if name not in "QT" else [21, 1, 30]
     seqs, refs = tiny_migurax.clear_sequences(name, _weights(name), lengths, min_gap=0.15)
     tol = _tolerance(dtype, name, seqs, refs)
     page = tiny_migurax.PAGE_SIZES[name]

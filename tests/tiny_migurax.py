@@ -1,6 +1,7 @@
 """Tiny random-weight folders of the Migurax design for the tests: sizes chosen so that what could coincide does not
 (query/key size against value size, rotated against unrotated dimensions, the query latent against the cache row),
-with one head and with more heads than a tile has rows, with a router that picks one, some or all of its experts, with
+with one head and with more heads than a tile has rows, at sizes that the matrix-core kernels take (Q, R) and at sizes they leave
+to the general ones (P, S), with a router that picks one, some or all of its experts, with
 a dense feed-forward, and with a layer that has none."""
 import json
 from pathlib import Path
@@ -27,12 +28,17 @@ CONFIGS = {
     ]),
     "Q": dict(architecture="Migurax", vocab=131, width=72, postln_alpha=1.0, norm=dict(eps=3e-6), layers=[
         dict(type="mlstm", mixer=dict(heads=4, dim=70, vdim=130, gate_cap=14.0), mlp=_moe(24, 4, 4)),
-        dict(type="latent_attention", mixer=_latent(20, 16, 8, 16, 32, 40, 0.25, 20000.0), mlp=dict(kind="dense", ff=96)),
+        dict(type="latent_attention", mixer=_latent(20, 16, 64, 16, 64, 40, 0.25, 20000.0), mlp=dict(kind="dense", ff=96)),
     ]),
     "R": dict(architecture="Migurax", vocab=64, width=64, postln_alpha=3.0, norm=dict(eps=1e-6), layers=[
-        dict(type="latent_attention", mixer=_latent(4, 16, 16, 32, 64, 48, 0.18, 1000.0), mlp=_moe(32, 8, 3)),
+        dict(type="latent_attention", mixer=_latent(4, 16, 32, 32, 128, 48, 0.18, 1000.0), mlp=_moe(32, 8, 3)),
         dict(type="mlstm", mixer=dict(heads=2, dim=32, vdim=64, gate_cap=10.0), mlp=_moe(32, 8, 3)),
-        dict(type="latent_attention", mixer=_latent(4, 16, 16, 32, 64, 48, 0.18, 1000.0), mlp=dict(kind="dense", ff=128)),
+        dict(type="latent_attention", mixer=_latent(4, 16, 32, 32, 128, 48, 0.18, 1000.0), mlp=dict(kind="dense", ff=128)),
+    ]),
+    # odd sizes everywhere: no width, rank or head size is a multiple of what the vectorised and matrix-core kernels want
+    "T": dict(architecture="Migurax", vocab=53, width=36, postln_alpha=2.5, norm=dict(eps=2e-5), layers=[
+        dict(type="latent_attention", mixer=_latent(2, 6, 2, 5, 10, 7, 0.4, 77.0), mlp=_moe(9, 2, 1)),
+        dict(type="mlstm", mixer=dict(heads=3, dim=5, vdim=7, gate_cap=6.0), mlp=dict(kind="dense", ff=11)),
     ]),
     # no routing, outputs at full strength, for tests in which far-away context must show in the logits
     "S": dict(architecture="Migurax", vocab=80, width=64, postln_alpha=1.0, norm=dict(eps=1e-5), layers=[
@@ -41,8 +47,8 @@ CONFIGS = {
         dict(type="latent_attention", mixer=_latent(2, 16, 16, 32, 32, 24, 0.25, 300.0), mlp=dict(kind="dense", ff=96)),
     ]),
 }
-SEEDS = {"P": 3, "Q": 4, "R": 6, "S": 8}
-PAGE_SIZES = {"P": 4, "Q": 16, "R": 8, "S": 16}
+SEEDS = {"P": 3, "Q": 4, "R": 6, "S": 8, "T": 9}
+PAGE_SIZES = {"P": 4, "Q": 16, "R": 8, "S": 16, "T": 2}
 
 
 def tensors_for(name: str, sharpen: float = 1.0) -> dict[str, torch.Tensor]:
