@@ -25,10 +25,13 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 // four groups of RPT rows side by side, which makes more and smaller work-groups where a step has few requests.
 // Tokens are taken TB at a time: their q, k, v go to shared memory, one wave turns their gates into decays (the capped
 // gates and the exponentials side by side, the running maximum one token after the other, as it is defined), every
-// lane runs the TB updates of its rows and leaves its rows' share of each token's sums, and the shares are added in the
-// order of the rows.  A share is always that of RPT rows whatever COLS is, so a token's result does not depend on how
-// the step was cut or on what else is in it.
+// lane runs the TB updates of its rows and leaves its rows' shares of each token's sums, and the shares are added in the
+// order of the rows.  A share is always that of four rows, whatever RPT and COLS are (a lane with RPT rows leaves RPT / 4
+// of them), so a token's result does not depend on how the step was cut or on what else is in it: a prompt is run with
+// few rows to a lane, because the time of a token is the chain of one lane's updates, a decode step with many rows and
+// wide tiles, because its time is the stream of the states.
 #define MLSTM_TB 16
+#define MLSTM_SHARE 4
 
 template <typename T, int RPT, int COLS>
 __global__ void __launch_bounds__(1024)
@@ -40,7 +43,8 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
     constexpr int RG = TL_WAVE / COLS;                 // groups of RPT rows a wave holds side by side
     extern __shared__ float smem[];
     const int waves = blockDim.x / TL_WAVE, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
-    const int shares = waves * RG;                     // ceil(dim / RPT)
+    constexpr int SPL = RPT / MLSTM_SHARE;             // shares of a lane
+    const int shares = waves * RG * SPL;               // >= ceil(dim / 4)
     // tb <= MLSTM_TB tokens are taken at a time: no more than the longest request of the step brings, so that a decode step's
     // work-groups need little shared memory and several fit a compute unit
     float* sq = smem;                                  // [tb][dim]
@@ -52,11 +56,11 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
     const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * (COLS - 1);
     const int tok0 = req_indptr[req], tok1 = req_indptr[req + 1];
     if (tok0 >= tok1) return;
-    const int c = lane % COLS, share = wave * RG + lane / COLS;
+    const int c = lane % COLS, share = (wave * RG + lane / COLS) * SPL;     // the first of this lane's shares
     const bool is_n = c == COLS - 1;
     const int col = col0 + c;
     const bool col_ok = !is_n && col < vdim;
-    const int row0 = share * RPT;
+    const int row0 = share * MLSTM_SHARE;
     float* st = state + (size_t)slots[req] * slot_stride + (size_t)head * ((size_t)dim * vdim + dim + 1);
     float* st_n = st + (size_t)dim * vdim;
     const float* nm = before + ((size_t)req * heads + head) * (dim + 1);      // n and m as they were before the launch
@@ -135,20 +139,17 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
             }
         }
         if (wave == 0) {
-            // the capped gates side by side, the running maximum token after token (every lane walks the same chain, the
-            // gates come from shared memory), then the decays side by side
+            // the capped gates side by side, the running maximum token after token (every lane walks the same chain),
+            // then the decays side by side
             const float gi = soft_cap(g_stage[0], cap), gf = log_sigmoid(soft_cap(g_stage[1], cap));
-            if (lane < nb) { sd[lane * 4 + 3] = gi; sd[lane * 4 + 2] = gf; }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             float m_before = m, m_mine = m;
-            for (int t = 0; t < nb; ++t) {
-                const float m_new = fmaxf(sd[t * 4 + 2] + m, sd[t * 4 + 3]);
+            for (int t = 0; t < nb; ++t) {             // (lane t's gates, read across the wave without a trip to shared memory)
+                const float fi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gi), t));
+                const float ff = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gf), t));
+                const float m_new = fmaxf(ff + m, fi);
                 if (lane == t) { m_before = m; m_mine = m_new; }
                 m = m_new;
             }
-            __builtin_amdgcn_wave_barrier();           // (every lane has read the gates before the maxima take their place)
             if (lane < nb) {
                 sd[lane * 4] = expf(gf + m_before - m_mine);
                 sd[lane * 4 + 1] = expf(gi - m_mine);
@@ -157,29 +158,41 @@ mlstm_scan_kernel(const T* __restrict__ qkv, int ld, int k_off, int v_off,
         }
         if (base + tb < tok1) fetch(base + tb);
         shared_barrier();
+#pragma unroll 4
         for (int t = 0; t < nb; ++t) {
             const float keep = sd[t * 4], tv = sd[t * 4 + 1] * sv[t * COLS + c];
             const float* kt = sk + t * dim + row0;
             const float* qt = sq + t * dim + row0;
-            float o = 0.f;
 #pragma unroll
-            for (int r = 0; r < RPT; ++r) {
-                if (row0 + r < dim) {
-                    S[r] = fmaf(kt[r], tv, keep * S[r]);
-                    o = fmaf(S[r], qt[r], o);
+            for (int u = 0; u < SPL; ++u) {
+                float o = 0.f;
+#pragma unroll
+                for (int r = MLSTM_SHARE * u; r < MLSTM_SHARE * (u + 1); ++r) {
+                    if (row0 + r < dim) {
+                        S[r] = fmaf(kt[r], tv, keep * S[r]);
+                        o = fmaf(S[r], qt[r], o);
+                    }
                 }
+                part[((size_t)t * shares + share + u) * COLS + c] = o;
             }
-            part[((size_t)t * shares + share) * COLS + c] = o;
         }
         shared_barrier();
         for (int t = wave; t < nb; t += waves) {
             if (lane < COLS) {
-                float osum = 0.f, nq = 0.f;
-                for (int w = 0; w < shares; ++w) {
-                    const float* p = part + ((size_t)t * shares + w) * COLS;
-                    osum += p[lane];
-                    nq += p[COLS - 1];
+                // the shares in four interleaved sums (shares 0, 4, 8, ...; 1, 5, 9, ...; ...), added up in their order:
+                // one fixed order whatever the work-group's shape, and four chains of additions instead of one
+                float o4[4] = {0.f, 0.f, 0.f, 0.f}, n4[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int w = 0; w < shares; w += 4) {          // (shares is a multiple of four or the tail is zeros of lanes without rows)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (w + u < shares) {
+                            const float* p = part + ((size_t)t * shares + w + u) * COLS;
+                            o4[u] += p[lane];
+                            n4[u] += p[COLS - 1];
+                        }
+                    }
                 }
+                const float osum = ((o4[0] + o4[1]) + o4[2]) + o4[3], nq = ((n4[0] + n4[1]) + n4[2]) + n4[3];
                 if (lane < COLS - 1 && col0 + lane < vdim)
                     out[((size_t)(base + t) * heads + head) * vdim + col0 + lane] = osum / (fmaxf(fabsf(nq), expf(-sd[t * 4 + 2])) + denom_eps);
             }
@@ -210,8 +223,9 @@ static int launch_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
                              const void* slots, const void* before, const void* req_indptr, void* out, int requests, int heads, int dim, int vdim,
                              float cap, float qscale, float denom_eps, int tb, hipStream_t stream) {
     constexpr int RG = TL_WAVE / COLS;
-    const int shares = (dim + RPT - 1) / RPT, waves = (shares + RG - 1) / RG;
-    const size_t smem = sizeof(float) * ((size_t)2 * tb * dim + tb * COLS + 4 * tb + (size_t)tb * waves * RG * COLS);
+    const int waves = (dim + RPT * RG - 1) / (RPT * RG);
+    TL_REQUIRE(waves <= 16, "mlstm_scan: %d rows of a head do not fit a work-group of %d rows a lane and %d columns", dim, RPT, COLS);
+    const size_t smem = sizeof(float) * ((size_t)2 * tb * dim + tb * COLS + 4 * tb + (size_t)tb * waves * RG * (RPT / MLSTM_SHARE) * COLS);
     TL_REQUIRE(smem <= 160 * 1024, "mlstm_scan: %zu bytes of shared memory for dim %d", smem, dim);
     auto kernel = mlstm_scan_kernel<T, RPT, COLS>;
     static size_t allowed = 48 * 1024;               // (per instance of the template)
@@ -245,11 +259,12 @@ extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
     TL_REQUIRE(slot_stride >= (long)heads * ((long)dim * vdim + dim + 1), "mlstm_scan: the state rows are too short");
     TL_REQUIRE(dtype == TL_DT_F32 || dtype == TL_DT_BF16, "mlstm_scan: unknown dtype %d", dtype);
     if (requests == 0) return TL_OK;
-    // rows a lane keeps: few for small heads (more waves at work), at most 16 shares of them to a work-group of 64 columns
-    const int rpt = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 256 ? 16 : dim <= 512 ? 32 : 64;
     // columns of a work-group: as few as it takes to give every compute unit one (the sums do not depend on the choice)
     const long heads_reqs = (long)heads * requests;
     const int cols = heads_reqs * ((vdim + 62) / 63) >= tl_mlstm_units ? 64 : heads_reqs * ((vdim + 30) / 31) >= tl_mlstm_units ? 32 : 16;
+    // rows a lane keeps: as few as 16 waves of such lanes can hold the head's rows with, four at least
+    const int need = (dim * cols + 16 * TL_WAVE - 1) / (16 * TL_WAVE);
+    const int rpt = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : need <= 32 ? 32 : 64;
 #define TL_MLSTM_C(R, C)                                                                                                       \
     return dtype == TL_DT_F32                                                                                                  \
         ? launch_mlstm_scan<float, R, C>(qkv, ld, k_off, v_off, gates, state, (size_t)slot_stride, slots, before, req_indptr, out,    \
