@@ -151,3 +151,20 @@ def test_trace_replay_reads_the_architecture_from_the_folder(cpu_ops, folders, t
     out = {s["step"]: np.fromfile(tmp_path / "out" / f"{s['step']}.f32", dtype="<f4").reshape(-1, 97) for s in steps
            if any(e["want"] for e in s["entries"])}
     scenarios.check(steps, out, refs, TOL, "trace replay")
+
+
+def test_command_line_writes_a_random_folder_of_the_architecture(tmp_path):
+    """``python -m torchlet_amd init`` from a Migurax config.json: the folder it writes declares the same layers, stores
+    every tensor the model declares under the design's names, and loads back through the registry."""
+    from safetensors import safe_open
+    from torchlet_amd.llm import main
+    from torchlet_amd.models.decoder import DecoderModel
+    src = tmp_path / "config.json"
+    src.write_text(json.dumps(tiny_migurax.CONFIGS["T"]))
+    assert main(["init", "--config", str(src), "--seed", "3", "--out", str(tmp_path / "out")]) == 0
+    cfg = load_config(tmp_path / "out")
+    assert isinstance(cfg, MiguraxConfig) and cfg.layers == tiny_migurax.CONFIGS["T"]["layers"] and cfg.postln_alpha == 2.5
+    with safe_open(str(tmp_path / "out" / "model.safetensors"), framework="pt") as f:
+        stored = set(f.keys())
+    assert stored == set(DecoderModel(cfg.to_spec(), torch.float32, "cpu").weight_specs())
+    assert {"embed", "head", "final.norm", "l0.mix.sink", "l0.mlp.router.b", "l1.mix.f.b", "l1.mlp.down.b"} <= stored
