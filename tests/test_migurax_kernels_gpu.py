@@ -59,7 +59,7 @@ def _plain_mlstm(q, k, v, gi, gf, cap, state):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim,cap", [(2, 40, 56, 12.0), (3, 20, 70, None), (1, 130, 96, 4.0), (2, 300, 130, 9.0)])
+@pytest.mark.parametrize("heads,dim,vdim,cap", [(2, 40, 56, 12.0), (3, 20, 70, None), (1, 130, 96, 4.0), (2, 300, 130, 9.0), (1, 700, 40, 5.0)])
 def test_mlstm_scan_portions_and_slots(dtype, heads, dim, vdim, cap):
     """Three requests in slots out of order, one of them continuing from a state that an earlier call left; a request's
     tokens in one call and the same tokens over two calls give the same outputs and the same state, bit for bit."""

@@ -225,7 +225,10 @@ static int launch_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
     constexpr int RG = TL_WAVE / COLS;
     const int waves = (dim + RPT * RG - 1) / (RPT * RG);
     TL_REQUIRE(waves <= 16, "mlstm_scan: %d rows of a head do not fit a work-group of %d rows a lane and %d columns", dim, RPT, COLS);
-    const size_t smem = sizeof(float) * ((size_t)2 * tb * dim + tb * COLS + 4 * tb + (size_t)tb * waves * RG * (RPT / MLSTM_SHARE) * COLS);
+    // tokens of a batch: as many as asked for, halved until their inputs and sums fit the shared memory (large heads)
+    const size_t per_token = sizeof(float) * ((size_t)2 * dim + COLS + 4 + (size_t)waves * RG * (RPT / MLSTM_SHARE) * COLS);
+    while (tb > 1 && per_token * tb > 144 * 1024) tb /= 2;
+    const size_t smem = per_token * tb;
     TL_REQUIRE(smem <= 160 * 1024, "mlstm_scan: %zu bytes of shared memory for dim %d", smem, dim);
     auto kernel = mlstm_scan_kernel<T, RPT, COLS>;
     static size_t allowed = 48 * 1024;               // (per instance of the template)
