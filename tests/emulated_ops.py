@@ -22,8 +22,37 @@ def load(names):
     pass
 
 
-def embedding(token_ids, table, out, scale=1.0):
-    out.copy_(table.float()[token_ids.long()] * scale)
+def embedding(token_ids, table, out, scale=1.0, positions=None, pos_table=None):
+    x = table.float()[token_ids.long()] * scale
+    if pos_table is not None:
+        x = x + pos_table.float()[positions.long()]
+    out.copy_(x if out.dim() == 2 else x[None].expand_as(out))
+
+
+MAX_STREAMS = 8
+
+
+def streams_norm(x, pending, fold, read, kind, weight, bias, eps, out, rows=None, gain=1.0):
+    S = x.shape[0]
+    new = x
+    if pending is not None:
+        p = pending.sum(0) if pending.dim() == 3 else pending.float()
+        if fold is None:
+            new = x + p[None]
+        else:
+            mix, gate = fold
+            new = torch.einsum("st,snw->tnw", mix, x) + gate[:, None, None] * p[None]
+    if rows is None:
+        x.copy_(new)
+    else:
+        new = new[:, rows.long()]
+    u = new.sum(0) if read is None else torch.einsum("s,snw->nw", read, new)
+    if kind == "layernorm":
+        mu = u.mean(-1, keepdim=True)
+        y = (u - mu) / torch.sqrt((u - mu).pow(2).mean(-1, keepdim=True) + eps) * weight.float() * gain + bias.float() * gain
+    else:
+        y = u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps) * gain * weight.float()
+    out.copy_(y.to(out.dtype))
 
 
 def add_rmsnorm(residual, pending, weight, eps, out, rows=None, gain=1.0):
@@ -224,16 +253,94 @@ def mlstm_scan(qkv, k_off, v_off, gates, state, slots, req_indptr, out, heads, d
         st[:, dim * vdim + dim] = m
 
 
-def gated_head_norm(o, gate, weight, eps, out, heads, vdim):
+def gated_head_norm(o, gate_values, weight, eps, out, heads, vdim, gate="sigmoid", gain=1.0):
     T = o.shape[0]
     x = o.view(T, heads, vdim)
-    y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
-    out.copy_((y.reshape(T, -1) * weight.float() * torch.sigmoid(gate.float())).to(out.dtype))
+    y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float().view(-1, vdim)
+    g = gate_values.float()
+    g = torch.sigmoid(g) if gate == "sigmoid" else g * torch.sigmoid(g)
+    out.copy_((y.reshape(T, -1) * g * gain).to(out.dtype))
+
+
+DELTA_MAX_TAPS = 8
+DELTA_MAX_DIM = 256
+LOCAL_ATTENTION_MAX_DIM = 256
+
+
+def delta_prepare(proj, conv_w, gates, a_log, dt_bias, state, tail_off, slots, req_indptr, token_req, qkv, heads, kv_heads, dim, vdim,
+                  taps, qscale, unit_eps):
+    C = 2 * kv_heads * dim + heads * vdim
+    for r in range(req_indptr.numel() - 1):
+        lo, hi = int(req_indptr[r]), int(req_indptr[r + 1])
+        if hi <= lo:
+            continue
+        st = state[int(slots[r])]
+        tail = st[tail_off: tail_off + (taps - 1) * C].view(taps - 1, C)
+        x = torch.cat((tail, proj[lo:hi, :C].float()), 0)                    # the inputs from taps - 1 tokens before the step on
+        y = sum(x[j: j + hi - lo] * conv_w[:, j] for j in range(taps))
+        y = y * torch.sigmoid(y)
+        qk = y[:, : 2 * kv_heads * dim].view(hi - lo, 2 * kv_heads, dim)
+        qk = qk / torch.sqrt(qk.pow(2).sum(-1, keepdim=True) + unit_eps)
+        qk[:, :kv_heads] *= qscale
+        qkv[lo:hi, : 2 * kv_heads * dim] = qk.reshape(hi - lo, -1)
+        qkv[lo:hi, 2 * kv_heads * dim:] = y[:, 2 * kv_heads * dim:]
+        if taps > 1:
+            tail.copy_(x[-(taps - 1):])
+    beta = torch.sigmoid(gates[:, :heads])
+    decay = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(gates[:, heads:] + dt_bias))
+    gates[:, :heads] = beta
+    gates[:, heads:] = decay
+
+
+def delta_scan(qkv, gates, state, slots, req_indptr, out, heads, kv_heads, dim, vdim, max_new_tokens=None):
+    of = torch.arange(heads) // (heads // kv_heads)
+    for r in range(req_indptr.numel() - 1):
+        st = state[int(slots[r])]
+        S = st[: heads * dim * vdim].view(heads, dim, vdim).clone()
+        for t in range(int(req_indptr[r]), int(req_indptr[r + 1])):
+            q = qkv[t, : kv_heads * dim].view(kv_heads, dim)[of]
+            k = qkv[t, kv_heads * dim: 2 * kv_heads * dim].view(kv_heads, dim)[of]
+            v = qkv[t, 2 * kv_heads * dim:].view(heads, vdim)
+            S = S * gates[t, heads:, None, None]
+            u = gates[t, :heads, None] * (v - torch.einsum("hde,hd->he", S, k))
+            S = S + k[:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hde,hd->he", S, q).reshape(-1)
+        st[: heads * dim * vdim] = S.reshape(-1)
+
+
+def kv_cache_write(k, v, token_req, positions, block_table, k_plane, v_plane, page_size):
+    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[3]
+    for t in range(k.shape[0]):
+        p = int(positions[t])
+        page = int(block_table[int(token_req[t]), p // page_size])
+        if page:
+            k_plane[page, :, p % page_size] = k[t].view(kv_heads, dim)
+            v_plane[page, :, p % page_size] = v[t].view(kv_heads, vdim)
+
+
+def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions, heads, kv_heads, dim, vdim, page_size, scale,
+                    softcap=0.0, chunk=0, window=0, gain=1.0, max_new_tokens=None, general=False):
+    group = heads // kv_heads
+    for t in range(q.shape[0]):
+        p, r = int(positions[t]), int(token_req[t])
+        lo = 0
+        if chunk:
+            lo = max(lo, p // chunk * chunk)
+        if window:
+            lo = max(lo, p - window + 1)
+        keys = torch.arange(lo, p + 1)
+        pages = block_table[r, keys // page_size].long()
+        k = k_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)      # [n, heads, dim]
+        v = v_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)
+        s = torch.einsum("hd,nhd->hn", q[t].float().view(heads, dim), k) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        out[t] = (torch.einsum("hn,nhd->hd", torch.softmax(s, -1), v).reshape(-1) * gain).to(out.dtype)
 
 
 LATENT_ATTENTION_ROWS = 16
 LATENT_MAX_RANK = 1024
-ACTIVATIONS = {"none": 0, "relu2": 1}
+ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19}
 
 
 LATENT_MFMA_ROWS = 64
@@ -316,7 +423,15 @@ def heads_linear(x, x_head, weight, out, out_head, general=False):
 
 
 def _act(y, activation):
-    return torch.clamp(y, min=0) ** 2 if activation == "relu2" else y
+    if activation.endswith("_pairs"):
+        return _act(y[:, 0::2], activation[: -len("_pairs")]) * y[:, 1::2]
+    if activation == "relu2":
+        return torch.clamp(y, min=0) ** 2
+    if activation == "silu":
+        return y * torch.sigmoid(y)
+    if activation == "gelu_tanh":
+        return 0.5 * y * (1 + torch.tanh(math.sqrt(2 / math.pi) * (y + 0.044715 * y ** 3)))
+    return y
 
 
 def experts_linear(x, slot_token, weight, offsets, out, activation="none", general=False):
@@ -327,10 +442,15 @@ def experts_linear(x, slot_token, weight, offsets, out, activation="none", gener
             out[lo:hi] = _act(rows.float() @ weight[e].float().T, activation).to(out.dtype)
 
 
-def route(logits, top):
+def route(logits, top, scores="chosen", choice_bias=None):
     T, E = logits.shape
-    best = logits.topk(top, dim=-1)               # ties: not met in tests
-    weights = torch.softmax(best.values, dim=-1)
+    if scores == "all":
+        s = torch.softmax(logits, dim=-1)
+        best = (s if choice_bias is None else s + choice_bias).topk(top, dim=-1)
+        weights = s.gather(1, best.indices)
+    else:
+        best = logits.topk(top, dim=-1)               # ties: not met in tests
+        weights = torch.softmax(best.values, dim=-1)
     chosen = best.indices.reshape(-1)
     order = torch.sort(chosen, stable=True).indices
     slot_token = (order // top).to(torch.int32)
@@ -341,9 +461,14 @@ def route(logits, top):
     return weights, offsets, slot_token, pair_slot
 
 
-def combine(y, pair_slot, weights, out):
+def combine(y, pair_slot, weights, out, identity=None):
     T, top = weights.shape
-    out.copy_((y[pair_slot.long()].float().view(T, top, -1) * weights[:, :, None]).sum(1).to(out.dtype))
+    rows = y[pair_slot.long()].float().view(T, top, -1)
+    if identity is not None:
+        x, offsets, experts = identity
+        own = (pair_slot >= offsets[experts]).view(T, top, 1)
+        rows = torch.where(own, x.float()[:, None, :], rows)
+    out.copy_((rows * weights[:, :, None]).sum(1).to(out.dtype))
 
 
 def activation(x, kind):

@@ -8,11 +8,12 @@ What it owns
   ``[runs, pages, heads, page_size, width]`` and one block table per request.
   A page id addresses every run and plane of its group, so one table row serves them all.  Page 0
   of every group is a sentinel that is never handed out and never written: empty table entries
-  point to it.  A group with a window needs fewer pages than one that keeps everything: when the
-  most tokens of a step are known its pool is sized for what its requests can hold at once.
+  point to it.  A group with a window (or with a mask in chunks) needs fewer pages than one that keeps
+  everything: when the most tokens of a step are known its pool is sized for what its requests can hold at once.
 * **Block tables.**  Per request and group, the list of pages in logical order.  A group
   with a window gives pages back as soon as every key in them lies behind the window of
-  all future queries; their table entries fall back to the sentinel.
+  all future queries (one with chunks: before the chunk of the next position); their table entries
+  fall back to the sentinel.
 * **Slots.**  A request holds one slot from admission to release.  Runs that declare a
   :class:`~torchlet_amd.parts.base.StateNeed` get a tensor ``[slots + 1, *shape]``; a slot's
   rows are zeroed when it is handed out.  The last row (``pad_slot``) belongs to no request: the
@@ -212,9 +213,9 @@ class CacheManager:
         """Most pages one request can hold in a group with a window when no step brings more than
         ``max_step_tokens`` tokens: the blocks from the first one a query can still read to the last
         one the step writes.  ``None``: no bound (no window, or steps of any size)."""
-        if need.window is None or self.max_step_tokens is None:
+        if not need.bounded or self.max_step_tokens is None:
             return None
-        return (need.window + self.max_step_tokens - 2) // self.page_size + 2
+        return (need.reach + self.max_step_tokens - 2) // self.page_size + 2
 
     def _pool_size(self, need: PagedNeed) -> int:
         most = self._held_at_most(need)
@@ -263,9 +264,12 @@ class CacheManager:
 
     def _first_live_block(self, g: _Group, length: int) -> int:
         """First logical block that a query at position >= ``length`` can still read."""
-        if g.need.window is None:
-            return 0
-        return max(0, length - g.need.window + 1) // self.page_size
+        first = 0
+        if g.need.window is not None:
+            first = max(first, length - g.need.window + 1)
+        if g.need.chunk is not None:          # the chunk that position `length` lies in starts here; later ones start later
+            first = max(first, length // g.need.chunk * g.need.chunk)
+        return first // self.page_size
 
     def pages_missing(self, req_id, new_length: int) -> list[int]:
         """Per group, the pages that ``reserve(req_id, new_length)`` would take.  (A request's
@@ -331,7 +335,7 @@ class CacheManager:
             raise CacheError(f"request {req_id!r} holds {r.length} tokens; cannot shrink to {new_length}")
         old_length, r.length = r.length, new_length
         for g in self.groups:
-            if g.need.window is None:
+            if not g.need.bounded:
                 continue
             table = g.tables[req_id]
             first = min(self._first_live_block(g, new_length), len(table))

@@ -37,6 +37,17 @@ class RMSNormSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class LayerNormSpec(PartSpec):
+    """``(x - mean) / sqrt(mean of squared deviations + eps) * weight + bias``.  ``weight_name`` / ``bias_name``: the two tensors
+    below the norm's own name; an empty ``weight_name``: the weight bears the norm's name itself."""
+    kind: ClassVar[str] = "layernorm"
+    dim: int = 0
+    eps: float = 1e-5
+    weight_name: str = "weight"
+    bias_name: str = "bias"
+
+
+@dataclass(frozen=True)
 class RotarySpec(PartSpec):
     """Split-half rotary position encoding over the whole head."""
     kind: ClassVar[str] = "rope_split_half"
@@ -112,6 +123,52 @@ class LatentAttentionSpec(PartSpec):
 
 
 @dataclass(frozen=True)
+class CappedAttentionSpec(PartSpec):
+    """Grouped-query attention over a paged cache whose keys and values differ in size (``dim`` and ``vdim`` per head), without a
+    position encoding of its own: ``score = q . k * scale``, then ``score <- softcap * tanh(score / softcap)`` (``None``: no cap);
+    query ``i`` reads the keys ``j <= i`` of its own chunk of ``chunk`` positions (chunks are counted from position 0; ``None``:
+    no chunks) and, with ``window``, the last ``window`` of them; an ordinary softmax; an output projection without bias."""
+    kind: ClassVar[str] = "capped_attention"
+    hidden: int = 0
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    scale: float = 1.0
+    softcap: float | None = None
+    chunk: int | None = None
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec(PartSpec):
+    """The gated delta rule: per head a ``dim x vdim`` state with ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``,
+    ``g = exp(-exp(A_log) softplus(W_a h + dt_bias))`` and ``beta = sigmoid(W_b h)`` per head; queries and keys (``kv_heads`` of them,
+    shared by ``heads / kv_heads`` heads each) and values pass a causal convolution of ``conv`` taps per channel and silu; queries and
+    keys are made unit vectors (``unit_eps`` under the root), queries times ``query_scale`` (``None``: ``dim ** -0.5``); each head's output is
+    divided by its root mean square (``norm_eps``), multiplied by one weight vector of ``vdim`` numbers and by ``silu(W_g h)``."""
+    kind: ClassVar[str] = "gated_delta"
+    hidden: int = 0
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    conv: int = 4
+    norm_eps: float = 1e-6
+    unit_eps: float = 1e-6
+    query_scale: float | None = None
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec(PartSpec):
+    """Several mixers side by side on the same input: ``sum_i scale_i * mixer_i(h)``.  ``branches``: ``(name, specification, scale)``
+    of each; ``name`` is the branch's sub-module name in the checkpoint."""
+    kind: ClassVar[str] = "parallel"
+    hidden: int = 0
+    branches: tuple = ()
+
+
+@dataclass(frozen=True)
 class DenseFFSpec(PartSpec):
     """``down(act(up(h)))`` with an elementwise activation (``relu2``: the square of relu) and optional biases."""
     kind: ClassVar[str] = "dense_ff"
@@ -123,8 +180,12 @@ class DenseFFSpec(PartSpec):
 
 @dataclass(frozen=True)
 class RoutedExpertsSpec(PartSpec):
-    """``experts`` small feed-forward layers ``down(act(up(h)))`` without biases; a linear router (with bias, in 32-bit)
-    picks the ``top`` largest logits per token, whose softmax (over the chosen ones only) weighs the experts' outputs."""
+    """``experts`` small feed-forward layers without biases, ``down(act(up(h)))`` or, ``gated``, ``down(act(gate(h)) * up(h))``; a linear
+    router (in 32-bit; ``router_bias``: with a bias) scores them, the ``top`` largest scores per token are chosen and weigh the chosen
+    experts' outputs.  ``scores``: ``"chosen"``: the choice goes by the logits and the weights are the softmax over the chosen ones alone;
+    ``"all"``: the scores are the softmax over all logits and the weights are the chosen experts' scores as they are.  ``choice_bias``: a
+    vector ``correction`` is added to the scores for the choice only.  ``identity``: the router has that many outputs beyond ``experts``;
+    an expert chosen among those returns its input."""
     kind: ClassVar[str] = "routed_experts"
     hidden: int = 0
     intermediate: int = 0
@@ -132,6 +193,10 @@ class RoutedExpertsSpec(PartSpec):
     top: int = 1
     activation: str = "relu2"
     router_bias: bool = True
+    gated: bool = False
+    scores: str = "chosen"
+    choice_bias: bool = False
+    identity: int = 0
 
 
 @dataclass(frozen=True)
@@ -157,6 +222,17 @@ class PostNormBlockSpec(BlockSpec):
     the sublayers read ``x`` itself.  ``ffn`` (and then ``ffn_norm``) may be ``None``: the layer ends after the first step."""
     kind: ClassVar[str] = "postnorm_residual"
     alpha: float = 1.0
+
+
+@dataclass(frozen=True)
+class HyperBlockSpec(BlockSpec):
+    """One layer over ``streams`` copies of the residual joined by hyper-connections.  Sublayer ``q`` (1: the mixer, 2: the
+    feed-forward) has a read vector ``in [streams]``, a matrix ``mix [streams, streams]`` (indexed from, to) and a write vector
+    ``out [streams]`` below ``connection_names[q - 1]``: ``u = sum_s in[s] x_s``, ``y = sublayer(norm(u))``, then all streams at once
+    ``x_t <- sum_s mix[s, t] x_s + out[t] y``.  ``ffn`` (and then ``ffn_norm``) may be ``None``."""
+    kind: ClassVar[str] = "hyper_connections"
+    streams: int = 1
+    connection_names: tuple = ("hc1", "hc2")
 
 
 @dataclass(frozen=True)
@@ -190,6 +266,8 @@ class ModelSpec:
     head_bias: bool = False        # the output head has a bias vector ``<head_name>.bias``
     weight_suffix: str = "weight"  # the embedding's and the head's matrix below their names; empty: the tensor bears the name itself
     layers_format: str = ""        # the name of layer i as a format string (``"l{}"``); empty: ``<layers_prefix>.<i>``
+    position_table_name: str = ""  # a learned table ``[max_positions, hidden]`` whose row of the position is added to the (scaled) embedding; empty: none
+    streams: int = 0               # copies of the residual that the blocks keep (hyper-connections); 0: the one plain residual
 
     def layer_name(self, i: int) -> str:
         return self.layers_format.format(i) if self.layers_format else f"{self.layers_prefix}.{i}"

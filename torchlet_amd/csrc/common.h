@@ -22,7 +22,7 @@ template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
 }
 
 // A vector (norm weight, bias) is stored either as bfloat16 or as float; read element i.
-__device__ __forceinline__ float load_vec(const void* p, int is_f32, int i) {
+__device__ __forceinline__ float load_vec(const void* p, int is_f32, size_t i) {
     return is_f32 ? ((const float*)p)[i] : to_float(((const bf16_t*)p)[i]);
 }
 

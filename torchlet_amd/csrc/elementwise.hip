@@ -4,27 +4,41 @@
 #include "common.h"
 
 // ------------------------------------------------------------------ embedding
-// out[t, :] = float(table[ids[t], :]) * scale; the residual stream is 32-bit.
+// out[c, t, :] = float(table[ids[t], :]) * scale (+ float(pos_table[positions[t], :])) for every copy c; the residual stream is 32-bit.
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                 float* __restrict__ out, int hidden, int vocab, float scale) {
+                                 float* __restrict__ out, int hidden, int vocab, float scale,
+                                 const int* __restrict__ positions, const void* __restrict__ pos_table, int pos_f32, int pos_rows,
+                                 int copies, size_t copy_stride) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= vocab) id = 0;  // ids are checked on the host; never read out of bounds
     const T* src = table + (size_t)id * hidden;
     float* dst = out + (size_t)t * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
+    int p = pos_table ? positions[t] : 0;
+    if (p < 0 || p >= pos_rows) p = 0;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = to_float(src[i]) * scale;
+        if (pos_table) v += load_vec(pos_table, pos_f32, (size_t)p * hidden + i);
+        for (int c = 0; c < copies; ++c) dst[c * copy_stride + i] = v;
+    }
 }
 
 extern "C" int tl_embedding(const void* ids, const void* table, int table_dtype, void* out,
-                            int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
+                            int tokens, int hidden, int vocab, float scale, const void* positions, const void* pos_table,
+                            int pos_dtype, int pos_rows, int copies, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0 && copies > 0, "embedding: bad sizes tokens=%d hidden=%d vocab=%d copies=%d", tokens, hidden, vocab, copies);
+    TL_REQUIRE(!pos_table || (positions && pos_rows > 0), "embedding: a position table needs positions and rows");
     if (tokens == 0) return TL_OK;
     dim3 grid(tokens), block(256);
+    const size_t copy_stride = (size_t)tokens * hidden;
+    const int pos_f32 = pos_dtype == TL_DT_F32;
     if (table_dtype == TL_DT_F32)
-        embedding_kernel<float><<<grid, block, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale);
+        embedding_kernel<float><<<grid, block, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale,
+                                                            (const int*)positions, pos_table, pos_f32, pos_rows, copies, copy_stride);
     else if (table_dtype == TL_DT_BF16)
-        embedding_kernel<bf16_t><<<grid, block, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale);
+        embedding_kernel<bf16_t><<<grid, block, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale,
+                                                             (const int*)positions, pos_table, pos_f32, pos_rows, copies, copy_stride);
     else TL_REQUIRE(false, "embedding: unknown dtype %d", table_dtype);
     TL_CHECK_LAUNCH("embedding");
     return TL_OK;
@@ -560,5 +574,106 @@ extern "C" int tl_scaled_add_rmsnorm(void* residual, const void* pending, int pa
         scaled_add_rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((float*)residual, pending, parts, part_stride, alpha, weight, weight_f32, eps, (bf16_t*)out, hidden);
     else TL_REQUIRE(false, "scaled_add_rmsnorm: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("scaled_add_rmsnorm");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ norm over several copies of the residual
+// x [S, T, hidden] float: S copies of the residual (hyper-connections).  One block per output row:
+//   the pending branch output p (one [T, hidden] tensor of the activation type, or `parts` float slabs of partial sums) enters
+//   all copies at once, x_t <- sum_s mix[s, t] x_s + gate[t] p (mix == null: x_t <- x_t + p), written back unless `rows` selects;
+//   u = sum_s read[s] x_s (read == null: the sum of the copies);
+//   kind 0: out = u / sqrt(mean(u^2) + eps) * gain * weight;  kind 1: out = ((u - mean) / sqrt(mean((u - mean)^2) + eps) * weight + bias) * gain.
+// u stays in shared memory between the passes (mean, squared deviations, output), so the deviations are taken from the mean itself.
+#define SN_MAX 8
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+streams_norm_kernel(float* __restrict__ x, int S, int total_rows, int hidden, const void* __restrict__ pending, int parts,
+                    const float* __restrict__ mix, const float* __restrict__ gate, const float* __restrict__ read, int kind,
+                    const void* __restrict__ weight, int weight_f32, const void* __restrict__ bias, int bias_f32, float eps, float gain,
+                    T* __restrict__ out, const int* __restrict__ rows) {
+    extern __shared__ float u_row[];                 // [hidden]
+    __shared__ float red[16];
+    const int orow = blockIdx.x;
+    const int srow = rows ? rows[orow] : orow;
+    const size_t copy_stride = (size_t)total_rows * hidden;
+    float* xr = x + (size_t)srow * hidden;
+    const T* pen = (pending && parts == 0) ? (const T*)pending + (size_t)srow * hidden : nullptr;
+    const float* slabs = (pending && parts > 0) ? (const float*)pending + (size_t)srow * hidden : nullptr;
+    const bool update = pending != nullptr && rows == nullptr;
+    float m[SN_MAX][SN_MAX], g[SN_MAX], rd[SN_MAX];
+#pragma unroll
+    for (int a = 0; a < SN_MAX; ++a) {
+        g[a] = (gate && a < S) ? gate[a] : 1.f;
+        rd[a] = a < S ? (read ? read[a] : 1.f) : 0.f;
+#pragma unroll
+        for (int b = 0; b < SN_MAX; ++b) m[a][b] = (mix && a < S && b < S) ? mix[a * S + b] : (a == b ? 1.f : 0.f);
+    }
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float xs[SN_MAX];
+#pragma unroll
+        for (int a = 0; a < SN_MAX; ++a) xs[a] = a < S ? xr[a * copy_stride + i] : 0.f;
+        float u = 0.f;
+        if (pending) {
+            float p = 0.f;
+            if (pen) p = to_float(pen[i]);
+            else
+                for (int q = 0; q < parts; ++q) p += slabs[q * copy_stride + i];
+#pragma unroll
+            for (int b = 0; b < SN_MAX; ++b) {
+                if (b < S) {
+                    float nb = 0.f;
+#pragma unroll
+                    for (int a = 0; a < SN_MAX; ++a)
+                        if (a < S) nb = fmaf(m[a][b], xs[a], nb);
+                    nb = fmaf(g[b], p, nb);
+                    if (update) xr[b * copy_stride + i] = nb;
+                    u = fmaf(rd[b], nb, u);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < SN_MAX; ++b)
+                if (b < S) u = fmaf(rd[b], xs[b], u);
+        }
+        u_row[i] = u;
+        sum += u;
+    }
+    float mean = 0.f;
+    if (kind == 1) mean = block_sum(sum, red) / (float)hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float d = u_row[i] - mean;
+        ss = fmaf(d, d, ss);
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)hidden + eps);
+    T* dst = out + (size_t)orow * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float d = (u_row[i] - mean) * inv;
+        const float w = load_vec(weight, weight_f32, i);
+        dst[i] = from_float<T>(kind == 1 ? (d * w + load_vec(bias, bias_f32, i)) * gain : d * gain * w);
+    }
+}
+
+extern "C" int tl_streams_norm(void* x, int streams, int total_rows, int hidden, const void* pending, int parts, const void* mix,
+                               const void* gate, const void* read, int kind, const void* weight, int weight_f32, const void* bias,
+                               int bias_f32, float eps, float gain, void* out, const void* rows, int n_out, int act_dtype, hipStream_t stream) {
+    TL_REQUIRE(streams >= 1 && streams <= SN_MAX && total_rows >= 0 && hidden > 0 && n_out >= 0, "streams_norm: bad sizes");
+    TL_REQUIRE(kind == 0 || (kind == 1 && bias), "streams_norm: kind %d (a layer norm needs its bias)", kind);
+    TL_REQUIRE((size_t)hidden * sizeof(float) <= 60 * 1024, "streams_norm: rows of %d numbers do not fit the shared memory", hidden);
+    TL_REQUIRE((mix == nullptr) == (gate == nullptr), "streams_norm: mix and gate come together");
+    if (n_out == 0) return TL_OK;
+    dim3 grid(n_out), block(256);
+    const size_t smem = (size_t)hidden * sizeof(float);
+    if (act_dtype == TL_DT_F32)
+        streams_norm_kernel<float><<<grid, block, smem, stream>>>((float*)x, streams, total_rows, hidden, pending, parts, (const float*)mix, (const float*)gate,
+                                                                  (const float*)read, kind, weight, weight_f32, bias, bias_f32, eps, gain, (float*)out, (const int*)rows);
+    else if (act_dtype == TL_DT_BF16)
+        streams_norm_kernel<bf16_t><<<grid, block, smem, stream>>>((float*)x, streams, total_rows, hidden, pending, parts, (const float*)mix, (const float*)gate,
+                                                                   (const float*)read, kind, weight, weight_f32, bias, bias_f32, eps, gain, (bf16_t*)out, (const int*)rows);
+    else TL_REQUIRE(false, "streams_norm: unknown dtype %d", act_dtype);
+    TL_CHECK_LAUNCH("streams_norm");
     return TL_OK;
 }

@@ -5,11 +5,18 @@
 
 #define ACT_NONE 0
 #define ACT_RELU2 1
+#define ACT_SILU 2
+#define ACT_GELU_TANH 3
+#define ACT_PAIRS 16      // added to one of the above: the product's columns 2i and 2i + 1 are a gate and an up value, the output act(gate) * up
 
 __device__ __forceinline__ float activate(float v, int act) {
     if (act == ACT_RELU2) { v = fmaxf(v, 0.f); return v * v; }
+    if (act == ACT_SILU) return v / (1.f + expf(-v));
+    if (act == ACT_GELU_TANH) return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
     return v;
 }
+
+__host__ __device__ __forceinline__ bool known_activation(int act) { return (act & ~ACT_PAIRS) >= ACT_NONE && (act & ~ACT_PAIRS) <= ACT_GELU_TANH; }
 
 // ------------------------------------------------------------------ grouped product
 // out[row(m), g_out + n] = act(sum_k a[src(m), g_a + k] * w[g][n][k]) for the rows m of group g, in tiles of 64 x 64
@@ -75,11 +82,20 @@ grouped_gemm_kernel(const T* __restrict__ a, int a_ld, int a_group, const int* _
         }
         __syncthreads();
     }
+    const int base_act = act & ~ACT_PAIRS;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = m0 + ty * 4 + i;
         if (m >= m_end) continue;
         T* orow = out + (size_t)m * out_ld + out_col;
+        if (act & ACT_PAIRS) {                          // (N is even: a pair lies in one thread's four columns)
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                const int n = n0 + tx * 4 + j;
+                if (n + 1 < N) orow[n / 2] = from_float<T>(activate(acc[i][j], base_act) * acc[i][j + 1]);
+            }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
@@ -157,6 +173,7 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ a, int a_ld, int a_group, co
         }
     }
     // acc[i][j][v] = out[row 16 j + li][column n0 + 16 i + 4 kg + v]
+    const int base_act = act & ~ACT_PAIRS;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int m = m0 + 16 * j + li;
@@ -165,6 +182,12 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ a, int a_ld, int a_group, co
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int n = n0 + 16 * i + 4 * kg;
+            if (act & ACT_PAIRS) {                      // a lane's four columns are two pairs: two outputs at column n / 2
+#pragma unroll
+                for (int v = 0; v < 4; v += 2)
+                    if (n + v + 1 < N) orow[(n + v) / 2] = from_float<bf16_t>(activate(acc[i][j][v], base_act) * acc[i][j][v + 1]);
+                continue;
+            }
             if (n + 3 < N && ((out_ld | out_col) & 3) == 0) {
                 union { uint2 u; uint16_t e[4]; } pk;
 #pragma unroll
@@ -182,7 +205,8 @@ grouped_gemm_mfma_kernel(const bf16_t* __restrict__ a, int a_ld, int a_group, co
 extern "C" int tl_grouped_gemm(const void* a, int a_ld, int a_group, const void* src, const void* w, void* out, int out_ld, int out_group,
                                const void* offsets, int groups, int rows, int N, int K, int act, int dtype, int general, hipStream_t stream) {
     TL_REQUIRE(groups > 0 && rows >= 0 && N > 0 && K > 0 && a_ld > 0 && out_ld > 0, "grouped_gemm: bad sizes");
-    TL_REQUIRE(act == ACT_NONE || act == ACT_RELU2, "grouped_gemm: unknown activation %d", act);
+    TL_REQUIRE(known_activation(act), "grouped_gemm: unknown activation %d", act);
+    TL_REQUIRE(!(act & ACT_PAIRS) || (N % 2 == 0 && out_group == 0), "grouped_gemm: an activation in pairs needs an even number of columns");
     if (rows == 0) return TL_OK;
     // with offsets, `rows` is the number of sorted slots in all groups together: every group may end in a partial tile
     dim3 grid(offsets ? (rows + GG_T - 1) / GG_T + groups : (rows + GG_T - 1) / GG_T, (N + GG_T - 1) / GG_T, offsets ? 1 : groups), block(256);
@@ -207,35 +231,48 @@ extern "C" int tl_grouped_gemm(const void* a, int a_ld, int a_group, const void*
 }
 
 // ------------------------------------------------------------------ the router's choice
-// Per token (one wave): the `top` largest of its `experts` logits, largest first (the lower index wins a tie), and
-// the softmax over those alone.
-__global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int* __restrict__ chosen,
-                                  float* __restrict__ weights, int tokens) {
+// Per token (one wave): the `top` best of its `experts` outputs, best first (the lower index wins a tie), and their weights.
+//   mode 0: the choice goes by the logits; the weights are the softmax over the chosen logits alone.
+//   mode 1: the scores are the softmax over all logits; the choice goes by score + bias[e] (bias optional), the weights are the
+//           chosen experts' scores as they are.
+__global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int mode, const float* __restrict__ bias,
+                                  int* __restrict__ chosen, float* __restrict__ weights, int tokens) {
     const int t = blockIdx.x * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     if (t >= tokens) return;
     const float* z = logits + (size_t)t * experts;
+    float zmax = 0.f, den = 1.f;
+    if (mode == 1) {
+        float mx = -INFINITY;
+        for (int e = lane; e < experts; e += TL_WAVE) mx = fmaxf(mx, z[e]);
+        zmax = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < experts; e += TL_WAVE) sum += expf(z[e] - zmax);
+        den = wave_sum(sum);
+    }
     float first = 0.f, sum = 0.f, mine = 0.f;           // lane j keeps the j-th choice's term
     unsigned long long taken = 0;                       // bit i: this lane's expert lane + 64 * i is chosen already
     for (int j = 0; j < top; ++j) {
-        float best = -INFINITY;
+        float best = -INFINITY, score = 0.f;
         int at = 0x7fffffff;
         for (int e = lane, i = 0; e < experts; e += TL_WAVE, ++i) {
-            const float v = z[e];
-            if (!((taken >> i) & 1ull) && (v > best || (v == best && e < at))) { best = v; at = e; }
+            float v = z[e], sc = 0.f;
+            if (mode == 1) { sc = expf(v - zmax) / den; v = bias ? sc + bias[e] : sc; }
+            if (!((taken >> i) & 1ull) && (v > best || (v == best && e < at))) { best = v; at = e; score = sc; }
         }
 #pragma unroll
         for (int o = TL_WAVE / 2; o > 0; o >>= 1) {
             const float ob = __shfl_xor(best, o, TL_WAVE);
+            const float os = __shfl_xor(score, o, TL_WAVE);
             const int oa = __shfl_xor(at, o, TL_WAVE);
-            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; score = os; }
         }
         if (at % TL_WAVE == lane) taken |= 1ull << (at / TL_WAVE);
         if (j == 0) first = best;
-        const float p = expf(best - first);
+        const float p = mode == 1 ? score : expf(best - first);
         sum += p;
         if (lane == j) { chosen[(size_t)t * top + j] = at; mine = p; }
     }
-    if (lane < top) weights[(size_t)t * top + lane] = mine / sum;
+    if (lane < top) weights[(size_t)t * top + lane] = mode == 1 ? mine : mine / sum;
 }
 
 // Sort of the (token, choice) pairs by expert, by one work-group: offsets[e] .. offsets[e + 1] - 1 are the slots of
@@ -260,12 +297,13 @@ route_sort_kernel(const int* __restrict__ chosen, int pairs, int top, int expert
     }
 }
 
-extern "C" int tl_route(const void* logits, int tokens, int experts, int top, void* chosen, void* weights, void* offsets,
-                        void* slot_token, void* pair_slot, hipStream_t stream) {
+extern "C" int tl_route(const void* logits, int tokens, int experts, int top, int mode, const void* bias, void* chosen, void* weights,
+                        void* offsets, void* slot_token, void* pair_slot, hipStream_t stream) {
+    TL_REQUIRE(mode == 0 || mode == 1, "route: unknown mode %d", mode);
     TL_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && top <= experts && top <= TL_WAVE && experts <= 64 * TL_WAVE, "route: bad sizes (experts %d, top %d)", experts, top);
     TL_REQUIRE((experts + 1) * sizeof(int) <= 64 * 1024, "route: too many experts (%d)", experts);
     if (tokens == 0) return TL_OK;
-    route_topk_kernel<<<(tokens + 3) / 4, 4 * TL_WAVE, 0, stream>>>((const float*)logits, experts, top, (int*)chosen, (float*)weights, tokens);
+    route_topk_kernel<<<(tokens + 3) / 4, 4 * TL_WAVE, 0, stream>>>((const float*)logits, experts, top, mode, (const float*)bias, (int*)chosen, (float*)weights, tokens);
     TL_CHECK_LAUNCH("route_topk");
     route_sort_kernel<<<1, 1024, (experts + 1) * sizeof(int), stream>>>((const int*)chosen, tokens * top, top, experts, (int*)offsets,
                                                                        (int*)slot_token, (int*)pair_slot);
@@ -274,27 +312,34 @@ extern "C" int tl_route(const void* logits, int tokens, int experts, int top, vo
 }
 
 // ------------------------------------------------------------------ weighted sum of the chosen experts' outputs
-// out[t, :] = sum_j weights[t, j] * y[pair_slot[t * top + j], :], summed in the order of the choices.
+// out[t, :] = sum_j weights[t, j] * y[pair_slot[t * top + j], :], summed in the order of the choices.  With `x`: a pair whose slot is
+// offsets[real] or later chose an expert without tensors (an identity expert), and x[t, :] stands in for its row of y.
 template <typename T>
 __global__ void combine_kernel(const T* __restrict__ y, const int* __restrict__ pair_slot, const float* __restrict__ weights,
-                               T* __restrict__ out, int top, int width) {
+                               T* __restrict__ out, const T* __restrict__ x, const int* __restrict__ offsets, int real, int top, int width) {
     const int t = blockIdx.x;
+    const int own_from = x ? offsets[real] : 0x7fffffff;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float a = 0.f;
-        for (int j = 0; j < top; ++j)
-            a = fmaf(weights[(size_t)t * top + j], to_float(y[(size_t)pair_slot[(size_t)t * top + j] * width + i]), a);
+        for (int j = 0; j < top; ++j) {
+            const int slot = pair_slot[(size_t)t * top + j];
+            const float v = slot >= own_from ? to_float(x[(size_t)t * width + i]) : to_float(y[(size_t)slot * width + i]);
+            a = fmaf(weights[(size_t)t * top + j], v, a);
+        }
         out[(size_t)t * width + i] = from_float<T>(a);
     }
 }
 
-extern "C" int tl_combine(const void* y, const void* pair_slot, const void* weights, void* out, int tokens, int top, int width,
-                          int dtype, hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && top > 0 && width > 0, "combine: bad sizes");
+extern "C" int tl_combine(const void* y, const void* pair_slot, const void* weights, void* out, const void* x, const void* offsets, int real,
+                          int tokens, int top, int width, int dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && top > 0 && width > 0 && real >= 0 && (!x || offsets), "combine: bad sizes");
     if (tokens == 0) return TL_OK;
     if (dtype == TL_DT_F32)
-        combine_kernel<float><<<tokens, 256, 0, stream>>>((const float*)y, (const int*)pair_slot, (const float*)weights, (float*)out, top, width);
+        combine_kernel<float><<<tokens, 256, 0, stream>>>((const float*)y, (const int*)pair_slot, (const float*)weights, (float*)out, (const float*)x,
+                                                          (const int*)offsets, real, top, width);
     else if (dtype == TL_DT_BF16)
-        combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)y, (const int*)pair_slot, (const float*)weights, (bf16_t*)out, top, width);
+        combine_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)y, (const int*)pair_slot, (const float*)weights, (bf16_t*)out, (const bf16_t*)x,
+                                                           (const int*)offsets, real, top, width);
     else TL_REQUIRE(false, "combine: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("combine");
     return TL_OK;
@@ -308,7 +353,7 @@ __global__ void activation_kernel(T* __restrict__ x, size_t n, int act) {
 }
 
 extern "C" int tl_activation(void* x, long n, int act, int dtype, hipStream_t stream) {
-    TL_REQUIRE(n >= 0 && (act == ACT_NONE || act == ACT_RELU2), "activation: bad arguments");
+    TL_REQUIRE(n >= 0 && known_activation(act) && !(act & ACT_PAIRS), "activation: bad arguments");
     if (n == 0 || act == ACT_NONE) return TL_OK;
     const int blocks = (int)((n + 1023) / 1024 < 8192 ? (n + 1023) / 1024 : 8192);
     if (dtype == TL_DT_F32) activation_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, (size_t)n, act);

@@ -1,5 +1,5 @@
-// Recurrent mixers with a fixed-size state per request: the matrix-memory recurrence (mLSTM) and the
-// gated per-head norm of its output.  State, gates, decays and the output's quotient are float whatever the
+// Recurrent mixers with a fixed-size state per request: the matrix-memory recurrence (mLSTM), the gated delta rule behind its
+// short convolutions, and the gated per-head norm of their outputs.  State, gates, decays and the output's quotient are float whatever the
 // activation type; queries, keys and values come in the activation type as the projection left them.
 #include "common.h"
 
@@ -290,11 +290,13 @@ extern "C" int tl_mlstm_scan(const void* qkv, int ld, int k_off, int v_off, cons
 }
 
 // ------------------------------------------------------------------ gated per-head norm
-// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gate[t, h, :]); one wave per token and head.
+// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * gate(g[t, h, :]) * gain; one wave per token and head.
+// gate 0: sigmoid, 1: silu.  shared_weight: one vector of vdim numbers for all heads.  The rows of g and y may be longer than
+// heads * vdim (views into wider buffers).
 template <typename T>
 __global__ void gated_head_norm_kernel(const float* __restrict__ o, const T* __restrict__ gate, int gate_ld,
-                                       const void* __restrict__ weight, int weight_f32, float eps,
-                                       T* __restrict__ out, int rows, int heads, int vdim) {
+                                       const void* __restrict__ weight, int weight_f32, int shared_weight, float eps,
+                                       T* __restrict__ out, int out_ld, int rows, int heads, int vdim, int gate_kind, float gain) {
     const int row = blockIdx.x * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     if (row >= rows) return;
     const int t = row / heads, h = row % heads;
@@ -304,24 +306,299 @@ __global__ void gated_head_norm_kernel(const float* __restrict__ o, const T* __r
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
     const T* g = gate + (size_t)t * gate_ld + h * vdim;
-    T* dst = out + (size_t)row * vdim;
+    T* dst = out + (size_t)t * out_ld + h * vdim;
+    const int w0 = shared_weight ? 0 : h * vdim;
     for (int i = lane; i < vdim; i += TL_WAVE) {
         const float z = to_float(g[i]);
-        dst[i] = from_float<T>(src[i] * inv * load_vec(weight, weight_f32, h * vdim + i) * (1.f / (1.f + expf(-z))));
+        const float s = 1.f / (1.f + expf(-z));
+        dst[i] = from_float<T>(src[i] * inv * load_vec(weight, weight_f32, w0 + i) * (gate_kind == 1 ? z * s : s) * gain);
     }
 }
 
-extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, const void* weight, int weight_f32, float eps,
-                                  void* out, int tokens, int heads, int vdim, int dtype, hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0 && gate_ld >= heads * vdim, "gated_head_norm: bad sizes");
+extern "C" int tl_gated_head_norm(const void* o, const void* gate, int gate_ld, const void* weight, int weight_f32, int shared_weight, float eps,
+                                  void* out, int out_ld, int tokens, int heads, int vdim, int gate_kind, float gain, int dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0 && gate_ld >= heads * vdim && out_ld >= heads * vdim, "gated_head_norm: bad sizes");
+    TL_REQUIRE(gate_kind == 0 || gate_kind == 1, "gated_head_norm: unknown gate %d", gate_kind);
     if (tokens == 0) return TL_OK;
     const int rows = tokens * heads;
     dim3 grid((rows + 3) / 4), block(4 * TL_WAVE);
     if (dtype == TL_DT_F32)
-        gated_head_norm_kernel<float><<<grid, block, 0, stream>>>((const float*)o, (const float*)gate, gate_ld, weight, weight_f32, eps, (float*)out, rows, heads, vdim);
+        gated_head_norm_kernel<float><<<grid, block, 0, stream>>>((const float*)o, (const float*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
+                                                                  (float*)out, out_ld, rows, heads, vdim, gate_kind, gain);
     else if (dtype == TL_DT_BF16)
-        gated_head_norm_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)o, (const bf16_t*)gate, gate_ld, weight, weight_f32, eps, (bf16_t*)out, rows, heads, vdim);
+        gated_head_norm_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)o, (const bf16_t*)gate, gate_ld, weight, weight_f32, shared_weight, eps,
+                                                                   (bf16_t*)out, out_ld, rows, heads, vdim, gate_kind, gain);
     else TL_REQUIRE(false, "gated_head_norm: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("gated_head_norm");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ gated delta rule: what the recurrence reads
+// A token's convolved channels come in units: kv_heads query heads, kv_heads key heads (dim channels each), heads value heads (vdim
+// channels each); one wave per token and unit.  Channel c at the request's i-th token of the step:
+//   y = sum_j w[c][j] * x[i - (taps - 1) + j][c],   x[i'] = the projection of the step's token i' >= 0, else tail[taps - 1 + i'][c]
+//   (the slot's last taps - 1 inputs from before the step, oldest first; zero for a new request), then silu;
+//   query and key heads: y / sqrt(sum y^2 + unit_eps), queries times qscale.
+// One more unit per token turns the raw gates into beta = sigmoid(b) and decay = exp(-exp(a_log) * softplus(a + dt_bias)).
+#define DELTA_MAX_TAPS 8
+#define DELTA_UNIT_MAX 4        // channels a lane holds: heads of up to 256 channels
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+delta_prepare_kernel(const T* __restrict__ proj, int ld, const float* __restrict__ conv_w, float* __restrict__ gates,
+                     const float* __restrict__ a_log, const float* __restrict__ dt_bias, const float* __restrict__ state, size_t slot_stride,
+                     size_t tail_off, const int* __restrict__ slots, const int* __restrict__ req_indptr, const int* __restrict__ token_req,
+                     float* __restrict__ qkv, int heads, int kv_heads, int dim, int vdim, int taps, float qscale, float unit_eps) {
+    const int t = blockIdx.x, lane = threadIdx.x % TL_WAVE;
+    const int unit = blockIdx.y * (blockDim.x / TL_WAVE) + threadIdx.x / TL_WAVE;
+    const int units = 2 * kv_heads + heads;
+    if (unit > units) return;
+    if (unit == units) {                               // the gates of the token's heads
+        for (int h = lane; h < heads; h += TL_WAVE) {
+            float* g = gates + (size_t)t * 2 * heads;
+            const float b = g[h], a = g[heads + h];
+            g[h] = 1.f / (1.f + expf(-b));
+            g[heads + h] = expf(-expf(a_log[h]) * softplus_f(a + dt_bias[h]));
+        }
+        return;
+    }
+    const int C = 2 * kv_heads * dim + heads * vdim;
+    const bool is_v = unit >= 2 * kv_heads;
+    const int width = is_v ? vdim : dim;
+    const int c0 = is_v ? 2 * kv_heads * dim + (unit - 2 * kv_heads) * vdim : unit * dim;
+    const int req = token_req[t];
+    const int i = t - req_indptr[req];                 // the token's place in its request's portion
+    const float* tail = state + (size_t)slots[req] * slot_stride + tail_off;
+    float y[DELTA_UNIT_MAX];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < DELTA_UNIT_MAX; ++u) {
+        const int c = c0 + lane + u * TL_WAVE;
+        y[u] = 0.f;
+        if (lane + u * TL_WAVE < width) {
+            float acc = 0.f;
+            for (int j = 0; j < taps; ++j) {
+                const int back = i - (taps - 1) + j;   // the input's place in the portion
+                const float xv = back >= 0 ? to_float(proj[(size_t)(t - i + back) * ld + c]) : tail[(size_t)(taps - 1 + back) * C + c];
+                acc = fmaf(conv_w[(size_t)c * taps + j], xv, acc);
+            }
+            y[u] = silu_f(acc);
+            ss = fmaf(y[u], y[u], ss);
+        }
+    }
+    float factor = 1.f;
+    if (!is_v) {
+        ss = wave_sum(ss);
+        factor = 1.f / sqrtf(ss + unit_eps);
+        if (unit < kv_heads) factor *= qscale;
+    }
+#pragma unroll
+    for (int u = 0; u < DELTA_UNIT_MAX; ++u)
+        if (lane + u * TL_WAVE < width) qkv[(size_t)t * C + c0 + lane + u * TL_WAVE] = y[u] * factor;
+}
+
+// After the step the tail of a request holds the last taps - 1 inputs of its channels: of the step's tokens, and before those of the
+// old tail.  A thread owns a channel of a request and reads the old tail before it writes.
+template <typename T>
+__global__ void delta_tail_kernel(const T* __restrict__ proj, int ld, float* __restrict__ state, size_t slot_stride, size_t tail_off,
+                                  const int* __restrict__ slots, const int* __restrict__ req_indptr, int C, int taps) {
+    const int req = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int tok0 = req_indptr[req], n = req_indptr[req + 1] - tok0;
+    if (c >= C || n <= 0) return;
+    float* tail = state + (size_t)slots[req] * slot_stride + tail_off;
+    float old[DELTA_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < DELTA_MAX_TAPS - 1; ++j) old[j] = j < taps - 1 ? tail[(size_t)j * C + c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < DELTA_MAX_TAPS - 1; ++j) {
+        if (j < taps - 1) {
+            const int back = n - (taps - 1) + j;       // place in the portion of what becomes entry j
+            float v = 0.f;
+            if (back >= 0) v = to_float(proj[(size_t)(tok0 + back) * ld + c]);
+            else {
+#pragma unroll
+                for (int q = 0; q < DELTA_MAX_TAPS - 1; ++q)
+                    if (q == j + n) v = old[q];
+            }
+            tail[(size_t)j * C + c] = v;
+        }
+    }
+}
+
+extern "C" int tl_delta_prepare(const void* proj, int ld, const void* conv_w, void* gates, const void* a_log, const void* dt_bias, void* state,
+                                long slot_stride, long tail_off, const void* slots, const void* req_indptr, const void* token_req, void* qkv,
+                                int tokens, int requests, int heads, int kv_heads, int dim, int vdim, int taps, float qscale, float unit_eps,
+                                int dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "delta_prepare: bad sizes");
+    TL_REQUIRE(taps >= 1 && taps <= DELTA_MAX_TAPS, "delta_prepare: 1 to %d taps are built, not %d", DELTA_MAX_TAPS, taps);
+    TL_REQUIRE(dim <= DELTA_UNIT_MAX * TL_WAVE && vdim <= DELTA_UNIT_MAX * TL_WAVE, "delta_prepare: heads of up to %d channels are built", DELTA_UNIT_MAX * TL_WAVE);
+    const int C = 2 * kv_heads * dim + heads * vdim;
+    TL_REQUIRE(ld >= C && tail_off >= 0 && slot_stride >= tail_off + (long)(taps - 1) * C, "delta_prepare: rows or state too short");
+    TL_REQUIRE(dtype == TL_DT_F32 || dtype == TL_DT_BF16, "delta_prepare: unknown dtype %d", dtype);
+    if (tokens == 0 || requests == 0) return TL_OK;
+    const int units = 2 * kv_heads + heads + 1;
+    dim3 grid(tokens, (units + 3) / 4), block(4 * TL_WAVE);
+    dim3 tgrid((C + 255) / 256, requests), tblock(256);
+    if (dtype == TL_DT_F32) {
+        delta_prepare_kernel<float><<<grid, block, 0, stream>>>((const float*)proj, ld, (const float*)conv_w, (float*)gates, (const float*)a_log, (const float*)dt_bias,
+            (const float*)state, (size_t)slot_stride, (size_t)tail_off, (const int*)slots, (const int*)req_indptr, (const int*)token_req, (float*)qkv,
+            heads, kv_heads, dim, vdim, taps, qscale, unit_eps);
+        TL_CHECK_LAUNCH("delta_prepare");
+        if (taps > 1) delta_tail_kernel<float><<<tgrid, tblock, 0, stream>>>((const float*)proj, ld, (float*)state, (size_t)slot_stride, (size_t)tail_off,
+                                                                             (const int*)slots, (const int*)req_indptr, C, taps);
+    } else {
+        delta_prepare_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)proj, ld, (const float*)conv_w, (float*)gates, (const float*)a_log, (const float*)dt_bias,
+            (const float*)state, (size_t)slot_stride, (size_t)tail_off, (const int*)slots, (const int*)req_indptr, (const int*)token_req, (float*)qkv,
+            heads, kv_heads, dim, vdim, taps, qscale, unit_eps);
+        TL_CHECK_LAUNCH("delta_prepare");
+        if (taps > 1) delta_tail_kernel<bf16_t><<<tgrid, tblock, 0, stream>>>((const bf16_t*)proj, ld, (float*)state, (size_t)slot_stride, (size_t)tail_off,
+                                                                              (const int*)slots, (const int*)req_indptr, C, taps);
+    }
+    TL_CHECK_LAUNCH("delta_tail");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ gated delta rule: the recurrence
+// Per request and head a state S of dim x vdim numbers; per token, with the decay g, the step size beta, unit q (scaled) and k:
+//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q.
+// Column j of S needs only its own a_j = sum_r S[r][j] k[r] and b_j = sum_r S[r][j] q[r] (of the state before the decay) and k . q:
+//   u_j = beta (v_j - g a_j);   o_j = g b_j + (k . q) u_j;   S[r][j] <- g S[r][j] + k[r] u_j.
+// A lane owns DELTA_RPL rows of one column in registers for all tokens of the step; L = 1 .. 16 lanes (a power of two, fixed by dim
+// alone) share a column and add their sums by exchanging across the wave, always in the same order, so a token's result depends
+// neither on how its request was cut into steps nor on what else the step holds.  A wave has 64 / L columns, a work-group of four
+// waves four times that: neighbouring columns, so that the rows of the state are fetched in whole lines.  Tokens are taken TB at a
+// time: their q, k, v, beta and g go to shared memory (the next batch is fetched into registers while this one is worked on), every
+// lane runs the TB updates of its rows, and the outputs leave through shared memory.
+#define DELTA_RPL 16
+#define DELTA_TB 16
+
+__global__ void __launch_bounds__(256)
+delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, float* __restrict__ state, size_t slot_stride,
+                  const int* __restrict__ slots, const int* __restrict__ req_indptr, float* __restrict__ out,
+                  int heads, int kv_heads, int dim, int vdim, int L, int tb) {
+    extern __shared__ float smem[];
+    const int CW = TL_WAVE / L;                        // columns of a wave
+    const int cols = 4 * CW;                           // ... of the work-group
+    const int rows_pad = L * DELTA_RPL;                // >= dim
+    float* sq = smem;                                  // [tb][rows_pad]
+    float* sk = sq + tb * rows_pad;                    // [tb][rows_pad]
+    float* sv = sk + tb * rows_pad;                    // [tb][cols]
+    float* sg = sv + tb * cols;                        // [tb][2]: beta, decay
+    float* so = sg + tb * 2;                           // [tb][cols]
+    const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * cols;
+    const int tok0 = req_indptr[req], tok1 = req_indptr[req + 1];
+    if (tok0 >= tok1) return;
+    const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
+    const int rg = lane / CW, cw = lane % CW;          // the lane's group of rows and its column within the wave
+    const int col = col0 + wave * CW + cw, row0 = rg * DELTA_RPL;
+    const bool col_ok = col < vdim;
+    const int C = 2 * kv_heads * dim + heads * vdim;
+    const int qk_head = head / (heads / kv_heads);
+    const int q_at = qk_head * dim, k_at = kv_heads * dim + qk_head * dim, v_at = 2 * kv_heads * dim + head * vdim + col0;
+    float* st = state + (size_t)slots[req] * slot_stride + (size_t)head * dim * vdim;
+
+    float S[DELTA_RPL];
+#pragma unroll
+    for (int r = 0; r < DELTA_RPL; ++r) S[r] = (col_ok && row0 + r < dim) ? st[(size_t)(row0 + r) * vdim + col] : 0.f;
+
+    // a batch's numbers, fetched into registers one batch ahead: per token 2 * rows_pad of q and k (zeros beyond dim), cols of v, 2 gates
+    const int per_token = 2 * rows_pad + cols + 2;
+    constexpr int STAGE = (DELTA_TB * (2 * 16 * DELTA_RPL + 4 * TL_WAVE + 2) + 255) / 256;       // at most, per thread
+    float stage[STAGE];
+    auto fetch = [&](int base) {
+        const int nb = min(tb, tok1 - base);
+#pragma unroll
+        for (int j = 0; j < STAGE; ++j) {
+            const int idx = threadIdx.x + j * 256;
+            float v = 0.f;
+            if (idx < nb * per_token) {
+                const int t = idx / per_token, e = idx % per_token;
+                const float* row = qkv + (size_t)(base + t) * C;
+                if (e < rows_pad) v = e < dim ? row[q_at + e] : 0.f;
+                else if (e < 2 * rows_pad) v = e - rows_pad < dim ? row[k_at + e - rows_pad] : 0.f;
+                else if (e < 2 * rows_pad + cols) v = col0 + e - 2 * rows_pad < vdim ? row[v_at + e - 2 * rows_pad] : 0.f;
+                else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * rows_pad - cols) * heads + head];
+            }
+            stage[j] = v;
+        }
+    };
+    fetch(tok0);
+    for (int base = tok0; base < tok1; base += tb) {
+        const int nb = min(tb, tok1 - base);
+        __syncthreads();                               // the batch before has been worked on and its outputs have left
+#pragma unroll
+        for (int j = 0; j < STAGE; ++j) {
+            const int idx = threadIdx.x + j * 256;
+            if (idx < nb * per_token) {
+                const int t = idx / per_token, e = idx % per_token;
+                if (e < rows_pad) sq[t * rows_pad + e] = stage[j];
+                else if (e < 2 * rows_pad) sk[t * rows_pad + e - rows_pad] = stage[j];
+                else if (e < 2 * rows_pad + cols) sv[t * cols + e - 2 * rows_pad] = stage[j];
+                else sg[t * 2 + e - 2 * rows_pad - cols] = stage[j];
+            }
+        }
+        if (base + tb < tok1) fetch(base + tb);
+        __syncthreads();
+        for (int t = 0; t < nb; ++t) {
+            const float* kt = sk + t * rows_pad + row0;
+            const float* qt = sq + t * rows_pad + row0;
+            float kr[DELTA_RPL], qr[DELTA_RPL];
+#pragma unroll
+            for (int r = 0; r < DELTA_RPL; r += 4) {
+                const float4 k4 = *(const float4*)(kt + r), q4 = *(const float4*)(qt + r);
+                kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
+                qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+            }
+            // four chains of additions each, joined in a fixed order
+            float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r = 0; r < DELTA_RPL; ++r) {
+                a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
+                b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
+                c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
+            }
+            float a = (a4[0] + a4[1]) + (a4[2] + a4[3]), b = (b4[0] + b4[1]) + (b4[2] + b4[3]), kq = (c4[0] + c4[1]) + (c4[2] + c4[3]);
+            for (int o = CW; o < TL_WAVE; o <<= 1) {   // the other groups of rows of this column
+                a += __shfl_xor(a, o, TL_WAVE);
+                b += __shfl_xor(b, o, TL_WAVE);
+                kq += __shfl_xor(kq, o, TL_WAVE);
+            }
+            const float beta = sg[t * 2], g = sg[t * 2 + 1];
+            const float u = beta * (sv[t * cols + wave * CW + cw] - g * a);
+#pragma unroll
+            for (int r = 0; r < DELTA_RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
+            if (rg == 0) so[t * cols + wave * CW + cw] = fmaf(kq, u, g * b);
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nb * cols; idx += 256) {
+            const int t = idx / cols, c = idx % cols;
+            if (col0 + c < vdim) out[((size_t)(base + t) * heads + head) * vdim + col0 + c] = so[idx];
+        }
+    }
+    if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < DELTA_RPL; ++r)
+            if (row0 + r < dim) st[(size_t)(row0 + r) * vdim + col] = S[r];
+    }
+}
+
+extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, long slot_stride, const void* slots, const void* req_indptr,
+                             void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
+    TL_REQUIRE(requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
+    TL_REQUIRE(dim <= 16 * DELTA_RPL, "delta_scan: built for up to %d query/key dimensions per head, got %d", 16 * DELTA_RPL, dim);
+    TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "delta_scan: the state rows are too short");
+    if (requests == 0) return TL_OK;
+    int L = 1;
+    while (L * DELTA_RPL < dim) L *= 2;
+    const int cols = 4 * (TL_WAVE / L);
+    const int tb = longest < 1 ? 1 : (longest < DELTA_TB ? longest : DELTA_TB);
+    const size_t smem = sizeof(float) * (size_t)tb * (2 * L * DELTA_RPL + 2 * cols + 2);
+    dim3 grid((vdim + cols - 1) / cols, heads, requests), block(256);
+    delta_scan_kernel<<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride, (const int*)slots,
+                                                     (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim, L, tb);
+    TL_CHECK_LAUNCH("delta_scan");
     return TL_OK;
 }

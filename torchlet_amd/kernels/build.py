@@ -47,6 +47,7 @@ def _targets(head_dims) -> dict[str, tuple[str, list[str]]]:
         "recurrent": ("recurrent.hip", []),
         "latent": ("latent.hip", []),
         "experts": ("experts.hip", []),
+        "local_attention": ("local_attention.hip", []),
     }
     for hd in head_dims:
         t[f"attention_hd{hd}"] = ("attention.hip", [f"-DTL_HEAD_DIM={hd}"])

@@ -120,16 +120,72 @@ def _i32(t: torch.Tensor | None, what: str, n: int | None = None) -> None:
 
 # ----------------------------------------------------------------------------- ops
 
-def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
-    """``out[t] = float(table[token_ids[t]]) * scale``; ``out`` is the 32-bit residual ``[T, H]``."""
+def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0,
+              positions: torch.Tensor | None = None, pos_table: torch.Tensor | None = None) -> None:
+    """``out[t] = float(table[token_ids[t]]) * scale (+ float(pos_table[positions[t]]))``; ``out`` is the 32-bit residual ``[T, H]``, or
+    ``[S, T, H]``: S copies of it."""
     T = token_ids.numel()
     V, H = table.shape
     _i32(token_ids, "embedding ids", T)
-    if out.shape != (T, H) or out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
-        raise KernelError(f"embedding: out must be contiguous float32 [{T}, {H}], got {out.dtype} {tuple(out.shape)}")
+    copies = out.shape[0] if out.dim() == 3 else 1
+    if out.shape[-2:] != (T, H) or out.dim() not in (2, 3) or out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
+        raise KernelError(f"embedding: out must be contiguous float32 [{T}, {H}] or [copies, {T}, {H}], got {out.dtype} {tuple(out.shape)}")
+    pos_rows = 0
+    if pos_table is not None:
+        _i32(positions, "embedding positions", T)
+        if positions is None or pos_table.dim() != 2 or pos_table.shape[1] != H or not pos_table.is_contiguous():
+            raise KernelError(f"embedding: a position table [rows, {H}] comes with the tokens' positions")
+        pos_rows = pos_table.shape[0]
     lib = _lib("elementwise")
     _check(lib, lib.tl_embedding(_ptr(token_ids), _ptr(table), c_int(_dt(table, "embedding table")), _ptr(out),
-                                 c_int(T), c_int(H), c_int(V), c_float(scale), _stream()))
+                                 c_int(T), c_int(H), c_int(V), c_float(scale), _ptr(positions if pos_rows else None),
+                                 _ptr(pos_table), c_int(_dt(pos_table, "position table") if pos_rows else 0), c_int(pos_rows),
+                                 c_int(copies), _stream()))
+
+
+NORM_KINDS = {"rmsnorm": 0, "layernorm": 1}
+MAX_STREAMS = 8
+
+
+def streams_norm(x: torch.Tensor, pending: torch.Tensor | None, fold, read: torch.Tensor | None, kind: str, weight: torch.Tensor,
+                 bias: torch.Tensor | None, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None, gain: float = 1.0) -> None:
+    """Over ``S`` copies of the residual, ``x`` float32 ``[S, T, H]``: the pending branch output ``p`` (``[T, H]`` of ``out``'s dtype, or
+    float32 slabs ``[P, T, H]`` of partial sums) enters all copies at once, ``x_t <- sum_s mix[s, t] x_s + gate[t] p`` with ``fold = (mix
+    [S, S], gate [S])`` float32 on the GPU (``fold=None``: ``x_t <- x_t + p``), then ``u = sum_s read[s] x_s`` (``read=None``: the sum of the
+    copies) and ``out = norm(u) * gain``: ``kind`` ``rmsnorm`` (``u / sqrt(mean(u^2) + eps) * weight``) or ``layernorm`` (``(u - mean) /
+    sqrt(mean((u - mean)^2) + eps) * weight + bias``).  Without ``rows`` the copies are updated in place; with ``rows`` (int32 source rows)
+    only those rows are read and nothing is written back."""
+    if x.dim() != 3 or x.dtype != torch.float32 or not x.is_contiguous() or not 1 <= x.shape[0] <= MAX_STREAMS:
+        raise KernelError(f"streams_norm: the residual copies must be contiguous float32 [S <= {MAX_STREAMS}, T, H], got {x.dtype} {tuple(x.shape)}")
+    S, T, H = x.shape
+    n = T if rows is None else rows.numel()
+    if out.shape != (n, H) or not out.is_contiguous():
+        raise KernelError(f"streams_norm: out must be contiguous [{n}, {H}], got {tuple(out.shape)}")
+    if kind not in NORM_KINDS or (kind == "layernorm") != (bias is not None):
+        raise KernelError(f"streams_norm: norm {kind!r} with{'out' if bias is None else ''} a bias is not built")
+    parts = 0
+    if pending is not None:
+        if pending.dim() == 3:
+            parts = pending.shape[0]
+            if pending.dtype != torch.float32 or pending.shape[1:] != (T, H) or not pending.is_contiguous():
+                raise KernelError(f"streams_norm: partial sums {pending.dtype} {tuple(pending.shape)} are not float32 [P, {T}, {H}]")
+        elif pending.shape != (T, H) or pending.dtype != out.dtype or not pending.is_contiguous():
+            raise KernelError(f"streams_norm: pending {pending.dtype} {tuple(pending.shape)} does not match [{T}, {H}] of {out.dtype}")
+    mix = gate = None
+    if fold is not None:
+        mix, gate = fold
+        if pending is None or mix.shape != (S, S) or gate.shape != (S,) or mix.dtype != torch.float32 or gate.dtype != torch.float32 \
+                or not mix.is_contiguous() or not gate.is_contiguous():
+            raise KernelError(f"streams_norm: a fold is float32 (mix [{S}, {S}], gate [{S}]) and comes with a pending output")
+    if read is not None and (read.shape != (S,) or read.dtype != torch.float32 or not read.is_contiguous()):
+        raise KernelError(f"streams_norm: read must be contiguous float32 [{S}]")
+    _i32(rows, "streams_norm rows")
+    wf = _vec(weight, H, "streams_norm weight")
+    bf = _vec(bias, H, "streams_norm bias")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_streams_norm(_ptr(x), c_int(S), c_int(T), c_int(H), _ptr(pending), c_int(parts), _ptr(mix), _ptr(gate), _ptr(read),
+                                    c_int(NORM_KINDS[kind]), _ptr(weight), c_int(wf), _ptr(bias), c_int(bf), c_float(eps), c_float(gain),
+                                    _ptr(out), _ptr(rows), c_int(n), c_int(_dt(out, "streams_norm")), _stream()))
 
 
 def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: torch.Tensor, eps: float,
@@ -780,18 +836,149 @@ def mlstm_scan(qkv: torch.Tensor, k_off: int, v_off: int, gates: torch.Tensor, s
                                   c_int(max(1, T - R + 1)), c_int(_dt(qkv, "mlstm_scan")), _stream()))
 
 
-def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, heads: int, vdim: int) -> None:
-    """``out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight[h] * sigmoid(gate[t, h])`` per token and head:
-    ``o`` float32 ``[T, heads * vdim]``, ``gate`` a row-strided view ``[T, heads * vdim]`` of ``out``'s dtype."""
+GATES = {"sigmoid": 0, "silu": 1}
+
+
+def gated_head_norm(o: torch.Tensor, gate_values: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, heads: int, vdim: int,
+                    gate: str = "sigmoid", gain: float = 1.0) -> None:
+    """``out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight[h] * gate(gate_values[t, h]) * gain`` per token and head:
+    ``o`` float32 ``[T, heads * vdim]``, ``gate_values`` and ``out`` row-strided views ``[T, heads * vdim]`` of one dtype; ``weight``
+    ``[heads * vdim]``, or ``[vdim]``: one vector for all heads; ``gate``: ``sigmoid`` or ``silu``."""
     T = o.shape[0]
     if o.dtype != torch.float32 or o.shape != (T, heads * vdim) or not o.is_contiguous():
         raise KernelError("gated_head_norm: o must be contiguous float32 [T, heads * vdim]")
-    if out.shape != o.shape or not out.is_contiguous() or gate.dtype != out.dtype or gate.shape != o.shape or gate.stride(1) != 1:
+    if out.shape != o.shape or out.stride(1) != 1 or gate_values.dtype != out.dtype or gate_values.shape != o.shape or gate_values.stride(1) != 1:
         raise KernelError("gated_head_norm: gate and out do not fit")
-    wf = _vec(weight, heads * vdim, "gated_head_norm weight")
+    shared = weight.numel() == vdim and heads > 1
+    wf = _vec(weight, vdim if shared else heads * vdim, "gated_head_norm weight")
     lib = _lib("recurrent")
-    _check(lib, lib.tl_gated_head_norm(_ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(wf), c_float(eps), _ptr(out),
-                                       c_int(T), c_int(heads), c_int(vdim), c_int(_dt(out, "gated_head_norm")), _stream()))
+    _check(lib, lib.tl_gated_head_norm(_ptr(o), _ptr(gate_values), c_int(gate_values.stride(0)), _ptr(weight), c_int(wf), c_int(1 if shared else 0),
+                                       c_float(eps), _ptr(out), c_int(out.stride(0)), c_int(T), c_int(heads), c_int(vdim), c_int(GATES[gate]),
+                                       c_float(gain), c_int(_dt(out, "gated_head_norm")), _stream()))
+
+
+# ------------------------------------------------------------- gated delta rule
+
+DELTA_MAX_TAPS = 8
+DELTA_MAX_DIM = 256
+
+
+def delta_prepare(proj: torch.Tensor, conv_w: torch.Tensor, gates: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                  state: torch.Tensor, tail_off: int, slots: torch.Tensor, req_indptr: torch.Tensor, token_req: torch.Tensor,
+                  qkv: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, taps: int, qscale: float, unit_eps: float) -> None:
+    """What the gated delta rule reads, made from the projections of the step's tokens.  ``proj [T, >= C]`` (a row-strided view) holds per
+    token the raw queries (``kv_heads * dim``), keys (the same) and values (``heads * vdim``), ``C`` channels in all.  Every channel passes
+    a causal convolution, ``y[t] = sum_j conv_w[c, j] x[t - (taps - 1) + j]``, whose inputs before the step's first token of a request
+    come from the request's slot (``state[slot, tail_off + i * C + c]``, ``i = 0 .. taps - 2`` oldest first), then silu; queries and keys
+    become unit vectors per head (``unit_eps`` under the root), queries times ``qscale``; the result goes to ``qkv`` float32 ``[T, C]``.
+    ``gates`` float32 ``[T, 2 * heads]`` holds the raw ``W_b h`` and ``W_a h`` and receives ``sigmoid(.)`` and ``exp(-exp(a_log) * softplus(. +
+    dt_bias))`` in their place.  Afterwards the slots' tails hold the last ``taps - 1`` inputs of every request."""
+    T = proj.shape[0]
+    R = req_indptr.numel() - 1
+    C = 2 * kv_heads * dim + heads * vdim
+    if proj.stride(1) != 1 or proj.shape[1] < C or qkv.dtype != torch.float32 or qkv.shape != (T, C) or not qkv.is_contiguous():
+        raise KernelError("delta_prepare: the projections or the output do not hold the convolved channels")
+    if conv_w.dtype != torch.float32 or conv_w.shape != (C, taps) or not conv_w.is_contiguous() or not 1 <= taps <= DELTA_MAX_TAPS:
+        raise KernelError(f"delta_prepare: taps must be contiguous float32 [{C}, {taps}], up to {DELTA_MAX_TAPS} of them")
+    if gates.dtype != torch.float32 or gates.shape != (T, 2 * heads) or not gates.is_contiguous():
+        raise KernelError(f"delta_prepare: gates must be contiguous float32 [{T}, {2 * heads}]")
+    for v, what in ((a_log, "a_log"), (dt_bias, "dt_bias")):
+        if v.dtype != torch.float32 or v.shape != (heads,) or not v.is_contiguous():
+            raise KernelError(f"delta_prepare: {what} must be contiguous float32 [{heads}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < tail_off + (taps - 1) * C:
+        raise KernelError(f"delta_prepare: state {tuple(state.shape)} does not hold the convolutions' tails")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    _i32(token_req, "token_req", T)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_delta_prepare(_ptr(proj), c_int(proj.stride(0)), _ptr(conv_w), _ptr(gates), _ptr(a_log), _ptr(dt_bias), _ptr(state),
+                                     ctypes.c_long(state.stride(0)), ctypes.c_long(tail_off), _ptr(slots), _ptr(req_indptr), _ptr(token_req),
+                                     _ptr(qkv), c_int(T), c_int(R), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(taps),
+                                     c_float(qscale), c_float(unit_eps), c_int(_dt(proj, "delta_prepare")), _stream()))
+
+
+def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, slots: torch.Tensor, req_indptr: torch.Tensor, out: torch.Tensor,
+               heads: int, kv_heads: int, dim: int, vdim: int, max_new_tokens: int | None = None) -> None:
+    """The gated delta rule over the step's tokens, request by request from the state its slot holds: ``qkv`` float32 ``[T, C]`` as
+    :func:`delta_prepare` left it (queries, keys, values), ``gates`` float32 ``[T, 2 * heads]`` (beta, decay); head ``h`` of ``state[slot]``
+    (float32, ``dim x vdim`` numbers from ``h * dim * vdim`` on) moves by ``S <- g S; u = beta (v - S^T k); S <- S + k u^T`` and ``out`` float32
+    ``[T, heads * vdim]`` receives ``S^T q``."""
+    T = qkv.shape[0]
+    R = req_indptr.numel() - 1
+    C = 2 * kv_heads * dim + heads * vdim
+    if qkv.dtype != torch.float32 or qkv.shape != (T, C) or not qkv.is_contiguous():
+        raise KernelError(f"delta_scan: qkv must be contiguous float32 [{T}, {C}]")
+    if gates.dtype != torch.float32 or gates.shape != (T, 2 * heads) or not gates.is_contiguous():
+        raise KernelError(f"delta_scan: gates must be contiguous float32 [{T}, {2 * heads}]")
+    if out.dtype != torch.float32 or out.shape != (T, heads * vdim) or not out.is_contiguous():
+        raise KernelError(f"delta_scan: out must be contiguous float32 [{T}, {heads * vdim}]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < heads * dim * vdim or dim > DELTA_MAX_DIM:
+        raise KernelError(f"delta_scan: state {tuple(state.shape)} does not hold {heads} states of {dim} x {vdim} (up to {DELTA_MAX_DIM} rows)")
+    _i32(slots, "slots", R)
+    _i32(req_indptr, "req_indptr", R + 1)
+    lib = _lib("recurrent")
+    _check(lib, lib.tl_delta_scan(_ptr(qkv), _ptr(gates), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(req_indptr), _ptr(out),
+                                  c_int(R), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim),
+                                  c_int(max(1, T - R + 1) if max_new_tokens is None else max_new_tokens), _stream()))
+
+
+# ------------------------------------------------------------- attention with two head sizes, a cap and a local mask
+
+LOCAL_ATTENTION_MAX_DIM = 256
+
+
+def _check_local_planes(what, k_plane, v_plane, dtype, kv_heads, dim, vdim, page_size):
+    if k_plane.dtype != dtype or v_plane.dtype != dtype or not k_plane.is_contiguous() or not v_plane.is_contiguous() \
+            or k_plane.shape[1:] != (kv_heads, page_size, dim) or v_plane.shape[1:] != (kv_heads, page_size, vdim) or k_plane.shape[0] != v_plane.shape[0]:
+        raise KernelError(f"{what}: cache planes {tuple(k_plane.shape)} / {tuple(v_plane.shape)} are not [pages, {kv_heads}, {page_size}, {dim} / {vdim}] of {dtype}")
+
+
+def kv_cache_write(k: torch.Tensor, v: torch.Tensor, token_req: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
+                   k_plane: torch.Tensor, v_plane: torch.Tensor, page_size: int) -> None:
+    """The step's keys ``k [T, kv_heads * dim]`` and values ``v [T, kv_heads * vdim]`` (row-strided views) go to their places in the pages:
+    token ``t`` of request ``token_req[t]`` at position ``p`` to slot ``p % page_size`` of page ``block_table[request, p // page_size]`` of
+    ``k_plane [pages, kv_heads, page_size, dim]`` and ``v_plane [pages, kv_heads, page_size, vdim]``.  What would go to page 0 is dropped."""
+    T = k.shape[0]
+    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[3]
+    _check_local_planes("kv_cache_write", k_plane, v_plane, k.dtype, kv_heads, dim, vdim, page_size)
+    if k.shape != (T, kv_heads * dim) or v.shape != (T, kv_heads * vdim) or k.stride(1) != 1 or v.stride(1) != 1 or v.dtype != k.dtype:
+        raise KernelError("kv_cache_write: keys or values do not fit the planes")
+    _i32(token_req, "token_req", T)
+    _i32(positions, "positions", T)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("kv_cache_write: the block table must be int32 [requests, blocks]")
+    lib = _lib("local_attention")
+    _check(lib, lib.tl_kv_cache_write(_ptr(k), c_int(k.stride(0)), _ptr(v), c_int(v.stride(0)), c_int(T), c_int(kv_heads), c_int(dim), c_int(vdim),
+                                      _ptr(token_req), _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]),
+                                      _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]), c_int(page_size), c_int(_dt(k, "kv_cache_write")), _stream()))
+
+
+def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch.Tensor,
+                    token_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, page_size: int,
+                    scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0,
+                    max_new_tokens: int | None = None, general: bool = False) -> None:
+    """Attention of the step's queries ``q [T, heads * dim]`` over their requests' cached keys and values (which hold the step's own tokens
+    already): query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then (``softcap > 0``) ``softcap *
+    tanh(score / softcap)``; a query at position ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (``chunk > 0``) and ``j > p -
+    window`` (``window > 0``); softmax and weighted sum in 32-bit; ``out [T, heads * vdim]`` receives the result times ``gain``.  ``q`` and ``out``
+    may be row-strided views.  ``max_new_tokens``: the most tokens a request brings in this step, if known (steps of single tokens skip
+    the kernel that tiles prompts); ``general=True`` forces the kernel without matrix cores."""
+    T = q.shape[0]
+    _check_local_planes("local_attention", k_plane, v_plane, q.dtype, kv_heads, dim, vdim, page_size)
+    if q.shape != (T, heads * dim) or out.shape != (T, heads * vdim) or q.stride(1) != 1 or out.stride(1) != 1 or out.dtype != q.dtype \
+            or heads % kv_heads or max(dim, vdim) > LOCAL_ATTENTION_MAX_DIM:
+        raise KernelError("local_attention: queries or output do not fit")
+    _i32(token_req, "token_req", T)
+    _i32(positions, "positions", T)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelError("local_attention: the block table must be int32 [requests, blocks]")
+    lib = _lib("local_attention")
+    _check(lib, lib.tl_local_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), c_int(out.stride(0)), _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]),
+                                       _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions),
+                                       c_int(T), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale),
+                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain),
+                                       c_int(T if max_new_tokens is None else max_new_tokens), c_int(1 if general else 0),
+                                       c_int(_dt(q, "local_attention")), _stream()))
 
 
 # ------------------------------------------------------------- attention over a cached latent
@@ -907,7 +1094,8 @@ def latent_attention(q: torch.Tensor, out: torch.Tensor, plane: torch.Tensor, bl
 
 # ------------------------------------------------------------- products over groups, routing
 
-ACTIVATIONS = {"none": 0, "relu2": 1}
+# ``*_pairs``: the product's columns come in pairs (gate, up) and the output, half as wide, is ``act(gate) * up``
+ACTIVATIONS = {"none": 0, "relu2": 1, "silu": 2, "gelu_tanh": 3, "relu2_pairs": 17, "silu_pairs": 18, "gelu_tanh_pairs": 19}
 
 
 def heads_linear(x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int, general: bool = False) -> None:
@@ -929,47 +1117,66 @@ def experts_linear(x: torch.Tensor, slot_token: torch.Tensor | None, weight: tor
                    activation: str = "none", general: bool = False) -> None:
     """``out[slot] = act(x[row(slot)] @ weight[e].T)`` for the slots ``offsets[e] .. offsets[e + 1] - 1`` of every expert ``e``;
     ``row(slot)`` is ``slot_token[slot]`` (a token routed to the expert) or, without it, the slot itself.  ``weight [experts, N, K]``,
-    ``out [slots, N]``."""
+    ``out [slots, N]``, or ``[slots, N / 2]`` for an activation in pairs (columns ``2i`` and ``2i + 1`` of the product give ``act(.) * .``).
+    Slots beyond ``offsets[experts]`` (of experts without tensors) are left alone."""
     G, N, K = weight.shape
     S = out.shape[0]
-    if x.dtype != weight.dtype or out.dtype != x.dtype or x.stride(1) != 1 or x.shape[1] != K or out.shape != (S, N) or not out.is_contiguous() \
-            or not weight.is_contiguous() or (slot_token is None and x.shape[0] != S):
+    pairs = ACTIVATIONS[activation] >= 16
+    if x.dtype != weight.dtype or out.dtype != x.dtype or x.stride(1) != 1 or x.shape[1] != K or out.shape != (S, N // 2 if pairs else N) \
+            or not out.is_contiguous() or not weight.is_contiguous() or (slot_token is None and x.shape[0] != S) or (pairs and N % 2):
         raise KernelError("experts_linear: shapes or dtypes do not fit")
     _i32(offsets, "offsets", G + 1)
     _i32(slot_token, "slot_token", S)
     lib = _lib("experts")
-    _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(0), _ptr(slot_token), _ptr(weight), _ptr(out), c_int(N), c_int(0),
+    _check(lib, lib.tl_grouped_gemm(_ptr(x), c_int(x.stride(0)), c_int(0), _ptr(slot_token), _ptr(weight), _ptr(out), c_int(out.shape[1]), c_int(0),
                                     _ptr(offsets), c_int(G), c_int(S), c_int(N), c_int(K), c_int(ACTIVATIONS[activation]),
                                     c_int(_dt(x, "experts_linear")), c_int(1 if general else 0), _stream()))
 
 
-def route(logits: torch.Tensor, top: int):
-    """The ``top`` largest logits of every row of float32 ``logits [T, experts]`` (the lower index wins a tie), the softmax over those
-    alone, and the sort of the (token, choice) pairs by expert: ``(weights [T, top] float32, offsets [experts + 1], slot_token [T * top],
-    pair_slot [T * top])``, all on the GPU: expert ``e`` owns the slots ``offsets[e] .. offsets[e + 1] - 1``, slot ``s`` reads token
-    ``slot_token[s]``, and the output row of token ``t``'s ``j``-th choice is ``pair_slot[t * top + j]``."""
+ROUTER_SCORES = {"chosen": 0, "all": 1}
+
+
+def route(logits: torch.Tensor, top: int, scores: str = "chosen", choice_bias: torch.Tensor | None = None):
+    """The router's choice for every row of float32 ``logits [T, experts]`` and the sort of the (token, choice) pairs by expert.
+    ``scores="chosen"``: the ``top`` largest logits are chosen and weighed by the softmax over those alone; ``"all"``: the scores are the
+    softmax over all logits, the ``top`` largest of score (+ ``choice_bias [experts]``, float32, which enters the choice only) are chosen
+    and weighed by their scores as they are.  The lower index wins a tie.  Returns ``(weights [T, top] float32, offsets [experts + 1],
+    slot_token [T * top], pair_slot [T * top])``, all on the GPU: expert ``e`` owns the slots ``offsets[e] .. offsets[e + 1] - 1``, slot
+    ``s`` reads token ``slot_token[s]``, and the output row of token ``t``'s ``j``-th choice is ``pair_slot[t * top + j]``."""
     T, E = logits.shape
     if logits.dtype != torch.float32 or not logits.is_contiguous() or not 0 < top <= min(E, 64) or E > 4096:
         raise KernelError("route: contiguous float32 logits, up to 4096 experts and up to 64 choices")
+    if choice_bias is not None and (choice_bias.dtype != torch.float32 or choice_bias.shape != (E,) or not choice_bias.is_contiguous()):
+        raise KernelError(f"route: the choice's bias must be contiguous float32 [{E}]")
     ints = torch.empty(T * top * 3 + E + 1, dtype=torch.int32, device=logits.device)
     chosen, slot_token, pair_slot, offsets = ints[: T * top], ints[T * top: 2 * T * top], ints[2 * T * top: 3 * T * top], ints[3 * T * top:]
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     lib = _lib("experts")
-    _check(lib, lib.tl_route(_ptr(logits), c_int(T), c_int(E), c_int(top), _ptr(chosen), _ptr(weights), _ptr(offsets), _ptr(slot_token),
-                             _ptr(pair_slot), _stream()))
+    _check(lib, lib.tl_route(_ptr(logits), c_int(T), c_int(E), c_int(top), c_int(ROUTER_SCORES[scores]), _ptr(choice_bias), _ptr(chosen), _ptr(weights),
+                             _ptr(offsets), _ptr(slot_token), _ptr(pair_slot), _stream()))
     return weights, offsets, slot_token, pair_slot
 
 
-def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[t] = sum_j weights[t, j] * y[pair_slot[t * top + j]]``, summed in 32-bit in the order of the choices."""
+def combine(y: torch.Tensor, pair_slot: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, identity=None) -> None:
+    """``out[t] = sum_j weights[t, j] * y[pair_slot[t * top + j]]``, summed in 32-bit in the order of the choices.  ``identity = (x,
+    offsets, experts)``: a pair whose slot is ``offsets[experts]`` or later chose an expert without tensors, and ``x[t]`` stands in for
+    its row of ``y``."""
     T, top = weights.shape
     W = out.shape[1]
     if y.shape != (T * top, W) or out.shape[0] != T or y.dtype != out.dtype or not y.is_contiguous() or not out.is_contiguous() \
             or weights.dtype != torch.float32 or not weights.is_contiguous():
         raise KernelError("combine: shapes or dtypes do not fit")
     _i32(pair_slot, "pair_slot", T * top)
+    x = offsets = None
+    experts = 0
+    if identity is not None:
+        x, offsets, experts = identity
+        if x.shape != (T, W) or x.dtype != out.dtype or not x.is_contiguous():
+            raise KernelError("combine: the input that stands in for identity experts does not fit")
+        _i32(offsets, "offsets", experts + 1)
     lib = _lib("experts")
-    _check(lib, lib.tl_combine(_ptr(y), _ptr(pair_slot), _ptr(weights), _ptr(out), c_int(T), c_int(top), c_int(W), c_int(_dt(out, "combine")), _stream()))
+    _check(lib, lib.tl_combine(_ptr(y), _ptr(pair_slot), _ptr(weights), _ptr(out), _ptr(x), _ptr(offsets), c_int(experts), c_int(T), c_int(top),
+                               c_int(W), c_int(_dt(out, "combine")), _stream()))
 
 
 def activation(x: torch.Tensor, kind: str) -> None:

@@ -1,6 +1,6 @@
 """A decoder built from a :class:`~torchlet_amd.config.base.ModelSpec`.
 
-embedding (times ``embed_scale``) -> the runs of the layer order -> final norm on the wanted rows
+embedding (times ``embed_scale``, plus the position's row of a learned table if the specification names one) -> the runs of the layer order -> final norm on the wanted rows
 (times ``logit_scale``) -> LM head (plus its bias, if the specification says it has one)
 (/root/reference/src/torchlet/v10_triton_paged_gqa/model/qwen2_5.py:55-87, where the factors are 1 and
 there is no bias).  The class
@@ -29,11 +29,14 @@ class DecoderModel:
         self.embed: torch.Tensor | None = None
         self.head: torch.Tensor | None = None
         self.head_bias: torch.Tensor | None = None
+        self.position_table: torch.Tensor | None = None
 
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> dict[str, WeightSpec]:
         s = self.spec
         specs = {join_name(s.embed_name, s.weight_suffix): WeightSpec((s.vocab_size, s.hidden))}
+        if s.position_table_name:
+            specs[join_name(s.position_table_name, s.weight_suffix)] = WeightSpec((s.max_positions, s.hidden), keep=KEEP_STORED)
         for i, block in enumerate(self.blocks):
             for k, v in block.weight_specs().items():
                 specs[join_name(s.layer_name(i), k)] = v
@@ -48,6 +51,8 @@ class DecoderModel:
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
         s = self.spec
         self.embed = place(tensors[join_name(s.embed_name, s.weight_suffix)], KEEP_COMPUTE, self.dtype, self.device)
+        if s.position_table_name:
+            self.position_table = place(tensors[join_name(s.position_table_name, s.weight_suffix)], KEEP_STORED, self.dtype, self.device)
         for i, block in enumerate(self.blocks):      # (`tensors` may read from disk on access: each name is touched once)
             block.load_weights(under(tensors, s.layer_name(i)))
         self.final_norm.load_weights(under(tensors, s.final_norm_name))
@@ -94,8 +99,11 @@ class DecoderModel:
         cache view of run ``i``.  Returns float32 logits ``[wanted rows, vocab]`` (``None``
         when no row is wanted)."""
         T = ctx.num_tokens
-        residual = torch.empty((T, self.spec.hidden), dtype=torch.float32, device=self.device)
-        ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale)
+        # the 32-bit residual, or the copies of it that blocks joined by hyper-connections keep: all start as the embedding's output
+        shape = (self.spec.streams, T, self.spec.hidden) if self.spec.streams else (T, self.spec.hidden)
+        residual = torch.empty(shape, dtype=torch.float32, device=self.device)
+        ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale,
+                      *((ctx.positions, self.position_table) if self.position_table is not None else ()))
         stream = Stream(residual)
         for i, e in enumerate(self.spec.order):
             stream = self.blocks[e.layer].forward(stream, ctx, caches[i])

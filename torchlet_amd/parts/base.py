@@ -57,6 +57,12 @@ def _init_one_plus_normal(shape, gen, device, std):
     return torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * std + 1.0
 
 
+@register_init_law("near_identity")
+def _init_near_identity(shape, gen, device, std):
+    """A square matrix: the identity plus N(0, std)."""
+    return torch.eye(shape[0], shape[1], device=device, dtype=torch.float32) + torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * std
+
+
 @register_init_law("random_table")
 def _init_random_table(shape, gen, device, std):
     return torch.randint(0, 2 ** 15, shape, generator=gen, device=device, dtype=torch.int32)
@@ -156,12 +162,26 @@ class PagedNeed:
     (``window=None``) or for the last ``window`` tokens.  ``planes`` is a count of planes of
     ``[num_heads, head_dim]`` each (keys and values are two), or a tuple of ``(heads, width)``, one per
     plane, for planes that differ (a compressed latent beside a small rotated part).  ``dtype``: the
-    planes' element type; ``None`` is the model's.  Layers with equal needs share a group of pages."""
+    planes' element type; ``None`` is the model's.  Layers with equal needs share a group of pages.  ``chunk``: a query reads only
+    keys of its own chunk of ``chunk`` positions (counted from position 0), so pages that lie wholly before the chunk of the next
+    position are kept no longer."""
     num_heads: int
     head_dim: int
     window: int | None = None
     planes: int | tuple[tuple[int, int], ...] = 2
     dtype: torch.dtype | None = None
+    chunk: int | None = None
+
+    @property
+    def bounded(self) -> bool:
+        """Whether a request keeps only a bounded stretch of its tokens (a window or a chunk)."""
+        return self.window is not None or self.chunk is not None
+
+    @property
+    def reach(self) -> int | None:
+        """Most positions back from a query that it can read, itself included (the smaller of window and chunk)."""
+        spans = [s for s in (self.window, self.chunk) if s is not None]
+        return min(spans) if spans else None
 
     @property
     def plane_shapes(self) -> tuple[tuple[int, int], ...]:
@@ -186,14 +206,19 @@ class Stream:
     of the last branch that is still to be added to it (``pending``, or ``None``).
     The next norm adds ``pending`` in 32-bit while it normalises, which saves one pass
     over the residual per branch.  ``pending`` is ``[T, hidden]`` in the activation dtype, or
-    float32 ``[P, T, hidden]``: P slabs of partial sums that the norm adds up as well."""
+    float32 ``[P, T, hidden]``: P slabs of partial sums that the norm adds up as well.
 
-    __slots__ = ("residual", "pending", "normed")
+    Blocks that keep several copies of the residual (hyper-connections) hold them as ``residual [S, T, hidden]``; ``fold`` then says
+    how the pending output enters them: ``(mix [S, S], out [S])``, 32-bit tensors on the GPU, for ``x_t <- sum_s mix[s, t] x_s +
+    out[t] * pending`` (``None``: ``pending`` is added to every stream as it is)."""
+
+    __slots__ = ("residual", "pending", "normed", "fold")
 
     def __init__(self, residual: torch.Tensor, pending: torch.Tensor | None = None):
         self.residual = residual
         self.pending = pending
         self.normed = None      # blocks whose norm follows the sum: the residual in the activation dtype, as the last norm left it
+        self.fold = None
 
 
 class LazyNorm:
@@ -238,11 +263,13 @@ class LazyNorm:
 # ----------------------------------------------------------------------- part kinds
 
 class Norm(Part):
-    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
         """Add ``stream.pending`` into ``stream.residual`` (both kept up to date) and
         return ``norm(residual) * gain`` in the activation dtype (the factor applied in 32-bit, before
         the one rounding of the result).  With ``rows`` (int32 indices) only those rows are read
-        and returned, and the stream is left untouched."""
+        and returned, and the stream is left untouched.  Over several copies of the residual (``residual [S, T, hidden]``) the
+        pending output enters through ``stream.fold`` and the norm reads ``sum_s read[s] x_s`` (``read``: 32-bit ``[S]`` on the GPU;
+        ``None``: the sum of the streams)."""
         raise NotImplementedError
 
     def renorm(self, stream: Stream, alpha: float = 1.0) -> torch.Tensor:
@@ -285,6 +312,43 @@ class Mixer(Part):
         :class:`torchlet_amd.cache.manager.LayerCache` (or ``None`` when the mixer
         declared no need)."""
         raise NotImplementedError
+
+
+class StagedMixer(Mixer):
+    """A mixer in three stages, so that it can also stand beside others on one input (``parallel``): an input projection
+    ``w_in [in_width, hidden]`` whose result it reads in the activation dtype, ``mix``, which turns that result into ``mix_width``
+    numbers per token, and an output projection ``w_o [hidden, mix_width]`` without bias.  A mixer of several such branches
+    stacks the ``w_in`` into one product and the ``w_o`` into another."""
+    in_width: int = 0
+    mix_width: int = 0
+    w_in: torch.Tensor | None = None
+    w_o: torch.Tensor | None = None
+
+    def mix(self, proj: torch.Tensor, h: torch.Tensor, ctx, cache, out: torch.Tensor, gain: float = 1.0) -> None:
+        """``proj [T, in_width]`` (a row-strided view of ``h @ w_in.T``) and ``h`` itself (for what the mixer projects on its own,
+        in 32-bit) -> ``out [T, mix_width]`` (a row-strided view), times ``gain``."""
+        raise NotImplementedError
+
+    def forward(self, h, ctx, cache):
+        from ..kernels import ops
+        T = h.shape[0]
+        proj = torch.empty((T, self.in_width), dtype=self.dtype, device=h.device)
+        ops.linear(h, self.w_in, None, proj)
+        mixed = torch.empty((T, self.mix_width), dtype=self.dtype, device=h.device)
+        self.mix(proj, h, ctx, cache, mixed)
+        return project_out(mixed, self.w_o, self.dtype)
+
+
+def project_out(mixed: torch.Tensor, w_o: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """A mixer's output projection ``[T, hidden]``, or (few rows against a narrow matrix, bfloat16) float32 slabs of partial sums
+    ``[P, T, hidden]`` that the next norm adds up."""
+    from ..kernels import ops
+    T, hidden = mixed.shape[0], w_o.shape[0]
+    if dtype == torch.bfloat16 and mixed.shape[1] % 64 == 0 and ops.linear_partials_pay(T, hidden, mixed.shape[1]):
+        return ops.linear_partials(mixed, w_o)
+    out = torch.empty((T, hidden), dtype=dtype, device=mixed.device)
+    ops.linear(mixed, w_o, None, out)
+    return out
 
 
 class FeedForward(Part):

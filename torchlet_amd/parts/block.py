@@ -8,10 +8,12 @@ adds it in 32-bit while it normalises.
 The other arrangement built here puts the norm after the sum: ``x <- norm1(alpha * x + mixer(x))``, then
 ``x <- norm2(alpha * x + ffn(x))``; the sublayers read the normed stream itself, and the sum and the norm are one
 kernel that leaves the stream in 32-bit and, for the products that read it next, in the activation dtype.
+
+A third one keeps several copies of the residual, joined by hyper-connections (:class:`HyperConnectionBlock`).
 """
 from __future__ import annotations
 
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, Stream, join_name, under
+from .base import BLOCKS, FEED_FORWARDS, KEEP_FLOAT32, MIXERS, NORMS, Block, Stream, WeightSpec, join_name, under
 
 
 @BLOCKS.register("prenorm_residual")
@@ -81,4 +83,55 @@ class PostNormBlock(Block):
             stream.pending = self.ffn.forward(h, ctx)
             h = self.ffn_norm.renorm(stream, self.alpha)
         stream.normed = h
+        return stream
+
+
+@BLOCKS.register("hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers over ``S`` copies of the residual, ``stream.residual [S, T, hidden]`` in 32-bit.  Sublayer ``q`` reads
+    ``u = sum_s in_q[s] x_s``, and its output ``y`` enters all copies at once, ``x_t <- sum_s mix_q[s, t] x_s + out_q[t] y``.  The
+    entry is deferred like the plain block's addition: the output is left pending on the stream with its ``(mix, out)``, and the
+    next norm's kernel (the block's second one, the next block's first one, the model's final one, which reads the sum of the
+    copies) does the entry, the read and the norm in one pass over the copies."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.streams = int(spec.streams)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.ffn = FEED_FORWARDS.build(spec.ffn, dtype, device) if spec.ffn is not None else None
+        self.ffn_norm = NORMS.build(spec.ffn_norm, dtype, device) if spec.ffn is not None else None
+        self._children = {spec.mixer_norm_name: self.mixer_norm, spec.mixer_name: self.mixer}
+        if self.ffn is not None:
+            self._children.update({spec.ffn_norm_name: self.ffn_norm, spec.ffn_name: self.ffn})
+        self.connections = list(spec.connection_names[: 2 if self.ffn is not None else 1])
+        self.read: list = []        # per sublayer: in [S]
+        self.fold: list = []        # per sublayer: (mix [S, S] indexed from, to; out [S])
+
+    parts = PreNormBlock.parts
+
+    def weight_specs(self):
+        S = self.streams
+        specs = PreNormBlock.weight_specs(self)
+        for name in self.connections:
+            specs[f"{name}.in"] = WeightSpec((S,), keep=KEEP_FLOAT32, init="one_plus_normal")
+            specs[f"{name}.out"] = WeightSpec((S,), keep=KEEP_FLOAT32, init="one_plus_normal")
+            specs[f"{name}.mix"] = WeightSpec((S, S), keep=KEEP_FLOAT32, init="near_identity")
+        return specs
+
+    def load_weights(self, tensors):
+        PreNormBlock.load_weights(self, tensors)
+        self.read = [self._place(tensors[f"{name}.in"], KEEP_FLOAT32) for name in self.connections]
+        self.fold = [(self._place(tensors[f"{name}.mix"], KEEP_FLOAT32), self._place(tensors[f"{name}.out"], KEEP_FLOAT32))
+                     for name in self.connections]
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        if stream.residual.dim() != 3 or stream.residual.shape[0] != self.streams:
+            raise ValueError(f"a block over {self.streams} copies of the residual got a stream of shape {tuple(stream.residual.shape)}")
+        h = self.mixer_norm.forward(stream, read=self.read[0])
+        stream.pending, stream.fold = self.mixer.forward(h, ctx, cache), self.fold[0]
+        if self.ffn is not None:
+            h = self.ffn_norm.forward(stream, read=self.read[1])
+            stream.pending, stream.fold = self.ffn.forward(h, ctx), self.fold[1]
         return stream

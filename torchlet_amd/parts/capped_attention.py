@@ -1,0 +1,63 @@
+"""Grouped-query attention with soft-capped scores and a mask in chunks, over a paged cache of keys and values of two sizes.
+
+``q = W_q h`` (``heads x dim``), ``k = W_k h`` (``kv_heads x dim``), ``v = W_v h`` (``kv_heads x vdim``), no biases and no position
+encoding; query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then ``score <- cap *
+tanh(score / cap)``; query ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (chunks are counted from position 0 of
+the sequence, whatever portion a step brings) and, with a window, ``j > p - window``; an ordinary softmax in 32-bit; ``W_o`` on the
+heads' values side by side.  The cache has two planes per page, ``[kv_heads, page, dim]`` and ``[kv_heads, page, vdim]``; pages that
+lie wholly before the chunk of a request's next position go back to the pool.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import ops
+from .base import KEEP_COMPUTE, MIXERS, PagedNeed, StagedMixer, WeightSpec
+
+
+@MIXERS.register("capped_attention")
+class CappedAttention(StagedMixer):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.heads % spec.kv_heads:
+            raise ConfigError(f"attention: {spec.heads} heads are not a multiple of {spec.kv_heads} key/value heads")
+        if spec.dim > ops.LOCAL_ATTENTION_MAX_DIM or spec.vdim > ops.LOCAL_ATTENTION_MAX_DIM:
+            raise ConfigError(f"attention kernels with two head sizes are built for up to {ops.LOCAL_ATTENTION_MAX_DIM} dimensions, not {spec.dim} / {spec.vdim}")
+        for name in ("chunk", "window"):
+            if getattr(spec, name) is not None and getattr(spec, name) < 1:
+                raise ConfigError(f"attention: a {name} must hold at least one key, got {getattr(spec, name)}")
+        self.hidden, self.heads, self.kv_heads, self.dim, self.vdim = spec.hidden, spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        self.q_width, self.k_width, self.v_width = spec.heads * spec.dim, spec.kv_heads * spec.dim, spec.kv_heads * spec.vdim
+        self.in_width = self.q_width + self.k_width + self.v_width
+        self.mix_width = spec.heads * spec.vdim
+        self.scale = float(spec.scale)
+        self.softcap = float(spec.softcap) if spec.softcap else 0.0
+        self.chunk, self.window = spec.chunk or 0, spec.window or 0
+
+    def paged_need(self):
+        return PagedNeed(num_heads=self.kv_heads, head_dim=self.dim, window=self.spec.window, chunk=self.spec.chunk,
+                         planes=((self.kv_heads, self.dim), (self.kv_heads, self.vdim)))
+
+    def kernel_libraries(self):
+        return ["local_attention"]
+
+    def weight_specs(self):
+        return {"q": WeightSpec((self.q_width, self.hidden)), "k": WeightSpec((self.k_width, self.hidden)),
+                "v": WeightSpec((self.v_width, self.hidden)), "o": WeightSpec((self.hidden, self.mix_width))}
+
+    def load_weights(self, tensors):
+        self.w_in = self._place(torch.cat([tensors[n] for n in "qkv"], dim=0), KEEP_COMPUTE)
+        self.w_o = self._place(tensors["o"], KEEP_COMPUTE)
+
+    def mix(self, proj, h, ctx, cache, out, gain=1.0):
+        k_plane, v_plane = cache.planes
+        table = ctx.block_tables[cache.group]
+        q = proj[:, : self.q_width]
+        if cache.writable:
+            ops.kv_cache_write(proj[:, self.q_width: self.q_width + self.k_width], proj[:, self.q_width + self.k_width:],
+                               ctx.token_req, ctx.positions, table, k_plane, v_plane, cache.page_size)
+        ops.local_attention(q, out, k_plane, v_plane, table, ctx.token_req, ctx.positions, self.heads, self.kv_heads, self.dim, self.vdim,
+                            cache.page_size, self.scale, self.softcap, self.chunk, self.window, gain, max_new_tokens=ctx.max_new_tokens)

@@ -7,6 +7,12 @@ the chosen ones alone, in 32-bit) weighs the experts' outputs ``W_down,e act(W_u
 of the choices.  The choice, the sort of the (token, choice) pairs by expert and the products over the experts' rows all
 happen on the GPU from device-side counts: nothing of a step's routing is read on the host, so decode steps can be
 recorded as graphs.
+
+The routed layer has other forms as well, each a field of its specification.  Gated experts, ``W_down,e (act(W_gate,e h) *
+W_up,e h)``: the rows of gate and up are interleaved into one matrix per expert and the product's epilogue applies the gate to
+each pair of neighbouring columns.  Scores over all experts: ``s = softmax(z)`` over every logit, the ``top`` largest of ``s +
+correction`` are chosen (the correction enters the choice only) and the weights are the chosen ``s`` as they are.  Identity
+experts: the router's last ``identity`` outputs have no tensors; a token that chooses one gets its own input times the weight.
 """
 from __future__ import annotations
 
@@ -65,20 +71,28 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
-        if not 0 < spec.top <= spec.experts:
-            raise ConfigError(f"a router picks between 1 and all of its experts, not {spec.top} of {spec.experts}")
         self.hidden, self.inter, self.experts, self.top = spec.hidden, spec.intermediate, spec.experts, spec.top
-        self.act = _activation(spec.activation)
-        self.w_router = self.b_router = self.w_up = self.w_down = None
+        self.identity = int(spec.identity)
+        self.outputs = self.experts + self.identity          # of the router
+        if not 0 < spec.top <= self.outputs:
+            raise ConfigError(f"a router picks between 1 and all of its experts, not {spec.top} of {self.outputs}")
+        if spec.scores not in ("chosen", "all"):
+            raise ConfigError(f"a router's scores are the softmax over the 'chosen' logits or over 'all', not {spec.scores!r}")
+        self.act = _activation(spec.activation + "_pairs" if spec.gated else spec.activation)
+        self.w_router = self.b_router = self.correction = self.w_up = self.w_down = None
 
     def kernel_libraries(self):
         return ["experts"]
 
     def weight_specs(self):
-        specs = {"router": WeightSpec((self.experts, self.hidden))}
+        specs = {"router": WeightSpec((self.outputs, self.hidden))}
         if self.spec.router_bias:
-            specs["router.b"] = WeightSpec((self.experts,), keep=KEEP_FLOAT32)
+            specs["router.b"] = WeightSpec((self.outputs,), keep=KEEP_FLOAT32)
+        if self.spec.choice_bias:
+            specs["correction"] = WeightSpec((self.outputs,), keep=KEEP_FLOAT32)
         for e in range(self.experts):
+            if self.spec.gated:
+                specs[f"e{e}.gate"] = WeightSpec((self.inter, self.hidden))
             specs[f"e{e}.up"] = WeightSpec((self.inter, self.hidden))
             specs[f"e{e}.down"] = WeightSpec((self.hidden, self.inter))
         return specs
@@ -86,18 +100,24 @@ class RoutedExperts(FeedForward):
     def load_weights(self, tensors):
         self.w_router = self._place(tensors["router"], KEEP_COMPUTE)
         self.b_router = self._place(tensors["router.b"], KEEP_FLOAT32) if self.spec.router_bias else None
-        self.w_up = self._place(torch.stack([tensors[f"e{e}.up"] for e in range(self.experts)]), KEEP_COMPUTE)
+        self.correction = self._place(tensors["correction"], KEEP_FLOAT32) if self.spec.choice_bias else None
+        if self.spec.gated:       # rows 2i and 2i + 1 of an expert's first matrix: row i of its gate and of its up
+            up = [torch.stack((tensors[f"e{e}.gate"], tensors[f"e{e}.up"]), dim=1).reshape(2 * self.inter, self.hidden) for e in range(self.experts)]
+        else:
+            up = [tensors[f"e{e}.up"] for e in range(self.experts)]
+        self.w_up = self._place(torch.stack(up), KEEP_COMPUTE)
         self.w_down = self._place(torch.stack([tensors[f"e{e}.down"] for e in range(self.experts)]), KEEP_COMPUTE)
 
     def forward(self, h, ctx):
         T = h.shape[0]
-        logits = torch.empty((T, self.experts), dtype=torch.float32, device=h.device)
+        logits = torch.empty((T, self.outputs), dtype=torch.float32, device=h.device)
         ops.linear(h, self.w_router, self.b_router, logits)
-        weights, offsets, slot_token, pair_slot = ops.route(logits, self.top)
+        weights, offsets, slot_token, pair_slot = ops.route(logits, self.top, self.spec.scores, self.correction)
         z = torch.empty((T * self.top, self.inter), dtype=self.dtype, device=h.device)
         ops.experts_linear(h, slot_token, self.w_up, offsets, z, self.act)
         y = torch.empty((T * self.top, self.hidden), dtype=self.dtype, device=h.device)
         ops.experts_linear(z, None, self.w_down, offsets, y)
         out = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
-        ops.combine(y, pair_slot, weights, out)
+        # (slots of identity experts lie behind those of the last expert with tensors: their rows of z and y are never written or read)
+        ops.combine(y, pair_slot, weights, out, identity=(h, offsets, self.experts) if self.identity else None)
         return out

@@ -10,7 +10,20 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import KEEP_STORED, NORMS, LazyNorm, Norm, Stream, WeightSpec
+from .base import KEEP_FLOAT32, KEEP_STORED, NORMS, LazyNorm, Norm, Stream, WeightSpec
+
+
+def _over_streams(kind: str, stream: Stream, weight, bias, eps: float, dtype, rows, gain: float, read) -> torch.Tensor:
+    """The norm ``kind`` of ``sum_s read[s] x_s`` over the copies of the residual, after the pending output has entered them
+    through ``stream.fold``: one kernel for the fold, the read and the norm.  A plain residual ``[T, hidden]`` is one stream."""
+    x = stream.residual if stream.residual.dim() == 3 else stream.residual.unsqueeze(0)
+    n = x.shape[1] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[2]), dtype=dtype, device=x.device)
+    ops.streams_norm(x, stream.pending, stream.fold, read, kind, weight, bias, eps, out, rows, gain)
+    if rows is None:
+        stream.pending = None
+        stream.fold = None
+    return out
 
 
 @NORMS.register("rmsnorm")
@@ -29,7 +42,9 @@ class RMSNorm(Norm):
     def load_weights(self, tensors):
         self.weight = self._place(tensors[self.spec.weight_name], KEEP_STORED)
 
-    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        if stream.residual.dim() == 3:
+            return _over_streams("rmsnorm", stream, self.weight, None, self.eps, self.dtype, rows, gain, read)
         n = stream.residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=self.dtype, device=stream.residual.device)
         ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, out, rows, gain)
@@ -49,6 +64,31 @@ class RMSNorm(Norm):
 
     def lazy(self, stream: Stream) -> LazyNorm | None:
         # one row in bfloat16: the kernels that read the norm's output can make it while their weights arrive
-        if self.dtype == torch.bfloat16 and stream.residual.shape[0] == 1 and stream.residual.is_cuda:
+        if self.dtype == torch.bfloat16 and stream.residual.dim() == 2 and stream.residual.shape[0] == 1 and stream.residual.is_cuda:
             return LazyNorm(self, stream, "rmsnorm", weight=self.weight, eps=self.eps)
         return None
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """``(r - mean(r)) / sqrt(mean((r - mean(r))^2) + eps) * weight + bias`` in 32-bit, fused with the entry of the pending branch
+    output into the residual (one plain residual, or several copies joined by hyper-connections)."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.dim = spec.dim
+        self.eps = float(spec.eps)
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def weight_specs(self):
+        return {self.spec.weight_name: WeightSpec((self.dim,), keep=KEEP_FLOAT32, init="one_plus_normal"),
+                self.spec.bias_name: WeightSpec((self.dim,), keep=KEEP_FLOAT32)}
+
+    def load_weights(self, tensors):
+        self.weight = self._place(tensors[self.spec.weight_name], KEEP_FLOAT32)
+        self.bias = self._place(tensors[self.spec.bias_name], KEEP_FLOAT32)
+
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0, read: torch.Tensor | None = None) -> torch.Tensor:
+        return _over_streams("layernorm", stream, self.weight, self.bias, self.eps, self.dtype, rows, gain, read)

@@ -10,6 +10,7 @@ from pathlib import Path
 
 from .config.base import ConfigError, ModelConfig
 from .config.migurax import MiguraxConfig
+from .config.nebutar import NebutarConfig
 from .config.qwen2 import Qwen2Config
 
 ARCHITECTURES: dict[str, type[ModelConfig]] = {}
@@ -28,6 +29,7 @@ def unregister_architecture(name: str) -> None:
 
 register_architecture(Qwen2Config)
 register_architecture(MiguraxConfig)
+register_architecture(NebutarConfig)
 
 
 def config_class(name: str) -> type[ModelConfig]:
