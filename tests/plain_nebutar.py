@@ -118,7 +118,9 @@ def parallel_mixer(h, w, m, eps):
 
 # ------------------------------------------------------------------ the feed-forward
 
-def routed_gated_experts(h, w, mlp, chosen_out=None):
+def routed_gated_experts(h, w, mlp, chosen_out=None, gaps=None):
+    """``gaps``: a list that receives, per token, how far the last chosen expert's choice score lies above the best one left out, as a
+    share of the two scores' sizes (about the difference of their logits)."""
     r = mlp["router"]
     E, ident, top = r["experts"], r.get("identity", 0), r["top"]
     s = torch.softmax(h @ w["router"].T, dim=-1)                  # over all experts, the identity ones included
@@ -126,6 +128,9 @@ def routed_gated_experts(h, w, mlp, chosen_out=None):
     idx = torch.topk(pick, top, dim=-1).indices
     if chosen_out is not None:
         chosen_out.append(idx)
+    if gaps is not None and top < E + ident:
+        ranked = torch.sort(pick, dim=-1, descending=True).values
+        gaps.extend(((ranked[:, top - 1] - ranked[:, top]) / (ranked[:, top - 1].abs() + ranked[:, top].abs())).tolist())
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e in idx[t].tolist():
@@ -153,9 +158,10 @@ def run_order(cfg):
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def forward(cfg, w, ids, layers_out=None, chosen_out=None):
+def forward(cfg, w, ids, layers_out=None, chosen_out=None, gaps=None, stored=lambda t: t):
     """Logits ``[n, vocab]`` of the whole sequence ``ids``.  ``layers_out``: a list that receives the sum of the streams after every
-    layer run."""
+    layer run.  ``stored``: applied to what the sublayers read and hand back (the tests round there, to see what reduced precision
+    between the parts does to the logits)."""
     dtype = w["embed"].dtype
     n = len(ids)
     eps = cfg["norm"]["eps"]
@@ -167,19 +173,19 @@ def forward(cfg, w, ids, layers_out=None, chosen_out=None):
         lw = sub(w, f"l{li}")
         assert layer["type"] == "parallel"
         for q, fn in ((1, lambda z: parallel_mixer(z, sub(lw, "mix"), layer["mixer"], eps)),
-                      (2, (lambda z: routed_gated_experts(z, sub(lw, "mlp"), layer["mlp"], chosen_out)) if layer.get("mlp") else None)):
+                      (2, (lambda z: routed_gated_experts(z, sub(lw, "mlp"), layer["mlp"], chosen_out, gaps)) if layer.get("mlp") else None)):
             if fn is None:
                 continue
             if S:
                 u = torch.einsum("s,snw->nw", lw[f"hc{q}.in"], xs)
             else:
                 u = xs[0]
-            y = fn(layer_norm(u, lw[f"norm{q}"], lw[f"norm{q}.b"], eps))
+            y = stored(fn(stored(layer_norm(u, lw[f"norm{q}"], lw[f"norm{q}.b"], eps))))
             if S:
                 xs = torch.einsum("st,snw->tnw", lw[f"hc{q}.mix"], xs) + lw[f"hc{q}.out"][:, None, None] * y[None]
             else:
                 xs = xs + y[None]
         if layers_out is not None:
             layers_out.append(xs.sum(0))
-    x = layer_norm(xs.sum(0), w["final.norm"], w["final.norm.b"], eps)
+    x = stored(layer_norm(xs.sum(0), w["final.norm"], w["final.norm.b"], eps))
     return (x @ w["embed"].T).to(dtype)
