@@ -81,13 +81,16 @@ def tensors_for(name: str, sharpen: float = 1.0) -> dict[str, torch.Tensor]:
             picks = torch.randperm(outputs, generator=g)[:top].tolist()
             for j, e in enumerate(picks):
                 code[t] += (1.0 - 0.3 * j) * directions[n][e]
+    routed_choices = any(outputs > top for outputs, top in routed.values())
     out = {}
     for k, v in random_tensors(cfg, SEEDS[name], torch.float32).items():
         tail = k.split(".", 1)[-1]
         if v.dim() == 2 and k not in ("embed", "pos") and not k.endswith((".conv", ".mix")) and ".hc" not in k:
             v = v * (50.0 / v.shape[1] ** 0.5)                  # N(0, 1 / fan_in)
         if k.endswith((".o", ".down")):
-            v = v * 0.2
+            v = v * (0.2 if routed_choices else 1.0)            # where no choice of experts hangs on it, the layers write at full strength
+        if k.endswith(".A_log") and not routed_choices:
+            v = torch.log(0.002 + 0.02 * torch.rand(v.shape, generator=g))      # slow decays: the state remembers hundreds of tokens
         if k == "embed":
             v = v * 15.0 + 1.2 * code
         if k == "pos":
