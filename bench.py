@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
                     [--shape 7b|14b|32b] [--context N] [--new-tokens G] [--prefill-tokens T]
-                    [--workload decode|serve|migurax] [--only decode|step|prefill] [--all]
+                    [--workload decode|serve|migurax|nebutar] [--only decode|step|prefill] [--all]
 
 The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV heads, head
 size 128, intermediate 18944, vocabulary 152064) with random weights and goes through the whole engine
@@ -39,6 +39,11 @@ with random weights: prefill of ``--prefill-tokens`` tokens in one step and deco
 caches (replayed graphs), beside a Qwen2 model of the same width, layer count and dense feed-forward width; and, under
 ``kernels``, every kernel that is the design's own alone at those sizes beside the like kernel of the Qwen2 path, each with
 the bytes it must move or the operations it must do and the fraction of the GPU's rate that this makes.
+
+``--workload nebutar [--size s|m]`` does the same for the Nebutar design (copies of the residual joined by hyper-connections; attention
+with soft-capped scores in chunks beside a gated delta rule; gated experts, some of them the identity), beside the Migurax model of
+the same width and layer count (the closest one the framework has: a recurrent state per request and routed experts), and its own
+kernels beside the like kernels of the Migurax and Qwen2 paths.
 """
 from __future__ import annotations
 
@@ -81,8 +86,8 @@ def parse_args(argv=None):
     p.add_argument("--context", type=int, default=CONTEXT, help="prompt tokens of each request in the decode runs")
     p.add_argument("--new-tokens", type=int, default=None, help="tokens each request may generate (decode: 256, serve: 128)")
     p.add_argument("--prefill-tokens", type=int, default=2048)
-    p.add_argument("--workload", choices=["decode", "serve", "migurax"], default="decode")
-    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax: layer sizes (s: width 2048, m: width 4096)")
+    p.add_argument("--workload", choices=["decode", "serve", "migurax", "nebutar"], default="decode")
+    p.add_argument("--size", choices=["s", "m"], default="s", help="migurax, nebutar: layer sizes (s: width 2048, m: width 4096)")
     p.add_argument("--requests", type=int, default=32)
     p.add_argument("--prompt-min", type=int, default=128)
     p.add_argument("--prompt-max", type=int, default=4096)
@@ -702,6 +707,200 @@ def migurax(args) -> dict:
     return out
 
 
+# ---------------------------------------------------------------------------------------------- the Nebutar design
+
+def nebutar_sizes(size: str) -> dict:
+    """A Nebutar configuration of four layers (the middle two form a span that runs once) at the width of the Migurax sizes: attention
+    heads of 128 + 128 in chunks of 1024, a delta rule with heads of 128 x 128 behind convolutions of four taps, gated experts."""
+    width, heads, experts, eff, top, streams = dict(s=(2048, 16, 16, 1024, 2, 4), m=(4096, 32, 32, 2048, 4, 4))[size]
+    left = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, softcap=30.0, mask=dict(size=1024))
+    right = dict(heads=heads, kv_heads=heads // 2, dim=128, vdim=128, conv=4)
+    layer = dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.7, right_scale=0.7),
+                 mlp=dict(kind="moe", expert=dict(ff=eff), router=dict(experts=experts, identity=2, top=top)))
+    return dict(architecture="Nebutar", vocab=32000, width=width, max_positions=8192, norm=dict(eps=1e-5), embedding=dict(scale=1.0),
+                streams=streams, loop=dict(start=1, stop=3, times=1), layers=[layer] * 4)
+
+
+def nebutar_kernels(ours: dict, like: dict, batch: int, context: int, tokens: int) -> list[dict]:
+    """Each kernel that is the design's own, alone, at the sizes of ``ours``, in a decode step of ``batch`` requests on ``context`` cached
+    tokens and in a prompt of ``tokens`` tokens, beside the like kernel of the Migurax or Qwen2 path.  ``frac``: bytes that must move /
+    time against 8 TB/s, or operations / time against the matrix cores' bfloat16 rate (against the 32-bit rate for the recurrences,
+    which the designs want in 32-bit)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, kind, launch, nbytes=0.0, flops=0.0, peak=MFMA_PEAK_TFLOPS["bfloat16"]):
+        ms = _best_ms(launch, rounds=3, calls=5)
+        row = {"kernel": name, "like": kind, "ms": round(ms, 4)}
+        if nbytes:
+            row.update(bytes=int(nbytes), frac=round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), bound="hbm")
+        else:
+            row.update(flops=flops, frac=round(flops / (ms * 1e-3) / (peak * 1e12), 4), bound="flops")
+        rows.append(row)
+        say(f"  {name}: {ms:.4f} ms, {row['frac']} of its bound")
+
+    def tables(n_req, total):
+        blocks = -(-total // PAGE)
+        table = (torch.arange(n_req * blocks, dtype=torch.int32, device=dev) + 1).view(n_req, blocks)
+        return table, n_req * blocks + 1
+
+    mixer, moe, width, S = ours["layers"][0]["mixer"], ours["layers"][0]["mlp"], ours["width"], ours["streams"]
+    left, right = mixer["left"], mixer["right"]
+    # ---- the delta rule beside the matrix-memory recurrence: a decode step reads and writes every state once; a prompt does 6 operations
+    #      per state element and token (two sums over the rows and the update), the matrix memory 4
+    h, g, d, v = right["heads"], right["kv_heads"], right["dim"], right["vdim"]
+    C = 2 * g * d + h * v
+    for name, T, reqs in (("delta_scan decode", batch, batch), (f"delta_scan prompt {tokens}", tokens, 1)):
+        qkv = torch.randn(T, C, device=dev) * 0.1
+        gates = torch.rand(T, 2 * h, device=dev) * 0.5 + 0.5
+        state = torch.zeros(reqs + 1, h * d * v, device=dev)
+        out = torch.empty(T, h * v, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        launch = lambda: ops.delta_scan(qkv, gates, state, slots, indptr, out, h, g, d, v, max_new_tokens=T // reqs)
+        if reqs > 1:
+            add(name, "mlstm_scan decode", launch, nbytes=2.0 * reqs * h * d * v * 4)
+        else:
+            add(name, f"mlstm_scan prompt {tokens}", launch, flops=6.0 * T * h * d * v, peak=MFMA_PEAK_TFLOPS["float32"])
+    rec = like["layers"][0]["mixer"]
+    mh, md, mv = rec["heads"], rec["dim"], rec["vdim"]
+    for name, T, reqs in (("mlstm_scan decode", batch, batch), (f"mlstm_scan prompt {tokens}", tokens, 1)):
+        qkv = torch.randn(T, 2 * mh * md + 2 * mh * mv, device=dev).to(bf)
+        gates = torch.randn(T, 2 * mh, device=dev)
+        state = torch.zeros(reqs + 1, mh, md * mv + md + 1, device=dev)
+        out = torch.empty(T, mh * mv, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        launch = lambda: ops.mlstm_scan(qkv, mh * md, 2 * mh * md, gates, state, slots, indptr, out, mh, md, mv, 12.0, md ** -0.5, 1e-6)
+        if reqs > 1:
+            add(name + " (Migurax path)", "", launch, nbytes=2.0 * reqs * mh * md * mv * 4)
+        else:
+            add(name + " (Migurax path)", "", launch, flops=4.0 * T * mh * md * mv, peak=MFMA_PEAK_TFLOPS["float32"])
+    # ---- what the delta rule reads: convolutions, silu, unit vectors, gates (reads the projections once, writes 32-bit numbers once)
+    for name, T, reqs in (("delta_prepare decode", batch, batch), (f"delta_prepare prompt {tokens}", tokens, 1)):
+        proj = torch.randn(T, C + h * v, device=dev).to(bf)
+        conv_w = torch.randn(C, right["conv"], device=dev)
+        gates = torch.randn(T, 2 * h, device=dev)
+        a_log, dt_bias = torch.zeros(h, device=dev), torch.zeros(h, device=dev)
+        state = torch.zeros(reqs + 1, (right["conv"] - 1) * C, device=dev)
+        slots = torch.arange(reqs, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(reqs + 1, dtype=torch.int32, device=dev) * (T // reqs))
+        token_req = torch.arange(T, dtype=torch.int32, device=dev) // (T // reqs)
+        out = torch.empty(T, C, device=dev)
+        launch = lambda: ops.delta_prepare(proj[:, :C], conv_w, gates, a_log, dt_bias, state, 0, slots, indptr, token_req, out, h, g, d, v, right["conv"], d ** -0.5, 1e-6)
+        add(name, "rope_cache_write", launch, nbytes=float(T) * C * (2 + 4) + 2.0 * reqs * (right["conv"] - 1) * C * 4)
+    # ---- attention with cap and chunks beside the Qwen2 path's attention: a decode step reads the cached keys and values it may see
+    #      once; a prompt's scores and sums (only inside the chunks)
+    H, G, dk, dv, chunk = left["heads"], left["kv_heads"], left["dim"], left["vdim"], left["mask"]["size"]
+    for name, T, reqs, ctx in (("local_attention decode", batch, batch, context - 1), (f"local_attention prompt {tokens}", tokens, 1, 0)):
+        total = ctx + T // reqs
+        table, pages = tables(reqs, total)
+        k_plane = (torch.randn(pages, G, PAGE, dk, device=dev) * 0.3).to(bf)
+        v_plane = (torch.randn(pages, G, dv, PAGE, device=dev) * 0.3).to(bf)
+        q = (torch.randn(T, H * dk, device=dev) * 0.3).to(bf)
+        out = torch.empty(T, H * dv, dtype=bf, device=dev)
+        token_req = torch.arange(T, dtype=torch.int32, device=dev) // (T // reqs)
+        positions = (torch.arange(T, dtype=torch.int32, device=dev) % (T // reqs)) + ctx
+        if reqs == 1:
+            n_tiles = -(-T // ops.LOCAL_ATTENTION_TILE_TOKENS)
+            tiles = (torch.tensor([0, T], dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev),
+                     torch.zeros(n_tiles, dtype=torch.int32, device=dev), torch.arange(n_tiles, dtype=torch.int32, device=dev) * ops.LOCAL_ATTENTION_TILE_TOKENS, n_tiles)
+        else:           # one token per request: a tile per request, no tile list
+            tiles = (torch.arange(reqs + 1, dtype=torch.int32, device=dev), torch.full((reqs,), ctx, dtype=torch.int32, device=dev), None, None, reqs)
+        launch = lambda: ops.local_attention(q, out, k_plane, v_plane, table, token_req, positions, H, G, dk, dv, PAGE, left["scale"], left["softcap"], chunk, 0, 0.7,
+                                             tiles=tiles)
+        if reqs > 1:
+            seen = ctx % chunk + 1                      # keys of the chunk the decoded token lies in
+            add(name, "paged_attention decode", launch, nbytes=float(reqs) * seen * G * (dk + dv) * 2)
+        else:
+            pairs = sum(p % chunk + 1 for p in range(T))
+            add(name, f"paged_attention_prompt {tokens}", launch, flops=2.0 * H * (dk + dv) * pairs)
+    qh, kvh, hd = H, G, 128
+    table, pages = tables(batch, context + 1)
+    k_plane = (torch.randn(pages, kvh, PAGE, hd, device=dev) * 0.3).to(bf)
+    v_plane = (torch.randn(pages, kvh, hd, PAGE, device=dev) * 0.3).to(bf)
+    q = (torch.randn(batch, qh * hd, device=dev) * 0.3).to(bf)
+    out = torch.empty(batch, qh * hd, dtype=bf, device=dev)
+    ctx_lens = torch.full((batch,), context, dtype=torch.int32, device=dev)
+    add("paged_attention decode (Qwen2 path)", "", lambda: ops.paged_attention(q, out, k_plane, v_plane, table, None, ctx_lens, None, None, batch, ops.attention_tile_tokens(qh, kvh), qh, kvh, hd, PAGE,
+                                                                              0, hd ** -0.5, 8, waves=8), nbytes=2.0 * batch * (context + 1) * kvh * hd * 2)
+    table, pages = tables(1, tokens)
+    k_plane = (torch.randn(pages, kvh, PAGE, hd, device=dev) * 0.3).to(bf)
+    v_plane = (torch.randn(pages, kvh, hd, PAGE, device=dev) * 0.3).to(bf)
+    q = (torch.randn(tokens, qh * hd, device=dev) * 0.3).to(bf)
+    out = torch.empty(tokens, qh * hd, dtype=bf, device=dev)
+    tq = ops.prompt_attention_tile_tokens(qh, kvh)
+    tiles = -(-tokens // tq)
+    tile_req = torch.zeros(tiles, dtype=torch.int32, device=dev)
+    tile_tok0 = torch.arange(tiles, dtype=torch.int32, device=dev) * tq
+    indptr = torch.tensor([0, tokens], dtype=torch.int32, device=dev)
+    zero = torch.zeros(1, dtype=torch.int32, device=dev)
+    add(f"paged_attention_prompt {tokens} (Qwen2 path)", "", lambda: ops.paged_attention_prompt(q, out, k_plane, v_plane, table, indptr, zero, tile_req, tile_tok0, tiles, tq,
+                                                                                                qh, kvh, hd, PAGE, 0, hd ** -0.5, max_total_len=tokens),
+        flops=float(qh) * 4 * hd * tokens * tokens / 2)
+    # ---- the norm over the copies of the residual beside the plain residual's norm: reads and writes every copy once
+    for name, T in (("streams_norm decode", batch), (f"streams_norm prompt {tokens}", tokens)):
+        x = torch.randn(S, T, width, device=dev)
+        pen = torch.randn(T, width, device=dev).to(bf)
+        fold = (torch.eye(S, device=dev), torch.ones(S, device=dev))
+        read = torch.ones(S, device=dev)
+        w, b = torch.ones(width, device=dev), torch.zeros(width, device=dev)
+        out = torch.empty(T, width, dtype=bf, device=dev)
+        add(name, "add_rmsnorm", lambda: ops.streams_norm(x, pen, fold, read, "layernorm", w, b, 1e-5, out), nbytes=float(T) * width * (8 * S + 4))
+        res = torch.randn(T, width, device=dev)
+        wb = torch.ones(width, dtype=bf, device=dev)
+        add(name.replace("streams_norm", "add_rmsnorm") + " (Qwen2 path)", "", lambda: ops.add_rmsnorm(res, pen, wb, 1e-5, out), nbytes=float(T) * width * 12)
+    # ---- the gated experts' first product (gate and up in pairs of columns) beside the Migurax path's (one matrix, squared relu)
+    E, top, ff = moe["router"]["experts"], moe["router"]["top"], moe["expert"]["ff"]
+    for name, T in (("experts_linear gated decode", batch), (f"experts_linear gated prompt {tokens}", tokens)):
+        x = torch.randn(T, width, device=dev).to(bf)
+        w_up = (torch.randn(E, 2 * ff, width, device=dev) * 0.02).to(bf)
+        logits = torch.randn(T, E + moe["router"]["identity"], device=dev)
+        weights, offsets, slot_token, pair_slot = ops.route(logits, top, "all", None)
+        z = torch.empty(T * top, ff, dtype=bf, device=dev)
+        real = int(offsets[E])
+        launch = lambda: ops.experts_linear(x, slot_token, w_up, offsets, z, "silu_pairs")
+        if T == batch:
+            add(name, "experts_linear decode", launch, nbytes=float(min(E, real)) * 2 * ff * width * 2)
+        else:
+            add(name, f"experts_linear prompt {tokens}", launch, flops=2.0 * real * 2 * ff * width)
+        w_one = (torch.randn(E, ff, width, device=dev) * 0.02).to(bf)
+        weights, offsets1, slot_token1, pair_slot = ops.route(torch.randn(T, E, device=dev), top)
+        launch = lambda: ops.experts_linear(x, slot_token1, w_one, offsets1, z, "relu2")
+        if T == batch:
+            add(name.replace(" gated", "") + " (Migurax path)", "", launch, nbytes=float(min(E, T * top)) * ff * width * 2)
+        else:
+            add(name.replace(" gated", "") + " (Migurax path)", "", launch, flops=2.0 * T * top * ff * width)
+    return rows
+
+
+def nebutar(args) -> dict:
+    import torch
+    ours = nebutar_sizes(args.size)
+    like, _ = migurax_sizes(args.size)
+    out = {"metric": f"Nebutar design, size {args.size} (width {ours['width']}, 4 layers), prefill of {args.prefill_tokens} tokens and decode at batch "
+                     f"{args.batch} on {args.context}-token caches, beside the Migurax design at equal width and layer count, one MI355X",
+           "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: seeded random weights, token ids and cache contents", "config": {"nebutar": ours, "migurax": like}}
+    for key, d in (("nebutar", ours), ("migurax", like)):
+        say(f"building the {key} model")
+        cfg, model = _build_from(d, args.dtype)
+        pms, pbest = time_prefill(model, args.prefill_tokens)
+        dms = _decode_ms(model, args.batch, min(args.steps, 64), args.warmup, args.context)
+        out[key] = {"weight_bytes": _weight_bytes(model),
+                    "prefill": {"tokens": args.prefill_tokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "tokens_per_s": round(args.prefill_tokens * 1e3 / pms, 1)},
+                    "decode": {"batch": args.batch, "context": args.context, "ms_per_step": round(dms, 4), "tokens_per_s": round(args.batch * 1e3 / dms, 1)}}
+        say(f"{key}: {out[key]}")
+        del model
+        torch.cuda.empty_cache()
+    out["value"] = out["nebutar"]["decode"]["tokens_per_s"]
+    if args.dtype == "bfloat16" and not args.no_points:
+        out["kernels"] = nebutar_kernels(ours, like, args.batch, args.context, args.prefill_tokens)
+    return out
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     args.serve_new_tokens = args.new_tokens or 128
@@ -715,6 +914,9 @@ def main(argv=None) -> int:
         return 1
     if args.workload == "migurax":
         print(json.dumps(migurax(args)))
+        return 0
+    if args.workload == "nebutar":
+        print(json.dumps(nebutar(args)))
         return 0
     name, sizes = SHAPES[args.shape]
     full_layers = sizes["num_hidden_layers"]

@@ -296,7 +296,7 @@ def delta_scan(qkv, gates, state, slots, req_indptr, out, heads, kv_heads, dim, 
     of = torch.arange(heads) // (heads // kv_heads)
     for r in range(req_indptr.numel() - 1):
         st = state[int(slots[r])]
-        S = st[: heads * dim * vdim].view(heads, dim, vdim).clone()
+        S = st[: heads * dim * vdim].view(heads, vdim, dim).transpose(1, 2).clone()          # a head's state lies column by column
         for t in range(int(req_indptr[r]), int(req_indptr[r + 1])):
             q = qkv[t, : kv_heads * dim].view(kv_heads, dim)[of]
             k = qkv[t, kv_heads * dim: 2 * kv_heads * dim].view(kv_heads, dim)[of]
@@ -305,21 +305,28 @@ def delta_scan(qkv, gates, state, slots, req_indptr, out, heads, kv_heads, dim, 
             u = gates[t, :heads, None] * (v - torch.einsum("hde,hd->he", S, k))
             S = S + k[:, :, None] * u[:, None, :]
             out[t] = torch.einsum("hde,hd->he", S, q).reshape(-1)
-        st[: heads * dim * vdim] = S.reshape(-1)
+        st[: heads * dim * vdim] = S.transpose(1, 2).reshape(-1)
 
 
 def kv_cache_write(k, v, token_req, positions, block_table, k_plane, v_plane, page_size):
-    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[3]
+    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[2]
     for t in range(k.shape[0]):
         p = int(positions[t])
         page = int(block_table[int(token_req[t]), p // page_size])
         if page:
             k_plane[page, :, p % page_size] = k[t].view(kv_heads, dim)
-            v_plane[page, :, p % page_size] = v[t].view(kv_heads, vdim)
+            v_plane[page, :, :, p % page_size] = v[t].view(kv_heads, vdim)
+
+
+LOCAL_ATTENTION_TILE_TOKENS = 16
+
+
+def local_attention_mfma_fits(dtype, dim, vdim, page_size):
+    return False
 
 
 def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions, heads, kv_heads, dim, vdim, page_size, scale,
-                    softcap=0.0, chunk=0, window=0, gain=1.0, max_new_tokens=None, general=False):
+                    softcap=0.0, chunk=0, window=0, gain=1.0, tiles=None):
     group = heads // kv_heads
     for t in range(q.shape[0]):
         p, r = int(positions[t]), int(token_req[t])
@@ -331,7 +338,7 @@ def local_attention(q, out, k_plane, v_plane, block_table, token_req, positions,
         keys = torch.arange(lo, p + 1)
         pages = block_table[r, keys // page_size].long()
         k = k_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)      # [n, heads, dim]
-        v = v_plane[pages, :, keys % page_size].float().repeat_interleave(group, dim=1)
+        v = v_plane[pages, :, :, keys % page_size].float().repeat_interleave(group, dim=1)
         s = torch.einsum("hd,nhd->hn", q[t].float().view(heads, dim), k) * scale
         if softcap:
             s = softcap * torch.tanh(s / softcap)

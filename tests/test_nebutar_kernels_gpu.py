@@ -80,13 +80,24 @@ def _paged(G, dim, vdim, page, lengths, dtype, g, scramble=True):
     order = (torch.randperm(pages - 1, generator=g) + 1).tolist() if scramble else list(range(1, pages))
     table = torch.zeros(len(lengths), max(blocks), dtype=torch.int32)
     k_plane = torch.full((pages, G, page, dim), float("nan")).to(dtype)
-    v_plane = torch.full((pages, G, page, vdim), float("nan")).to(dtype)
+    v_plane = torch.full((pages, G, vdim, page), float("nan")).to(dtype)            # the values of a page lie transposed
     keys = [torch.randn(n, G, dim, generator=g).to(dtype) for n in lengths]
     values = [torch.randn(n, G, vdim, generator=g).to(dtype) for n in lengths]
     for r, n in enumerate(lengths):
         for b in range(blocks[r]):
             table[r, b] = order.pop()
     return table, k_plane, v_plane, keys, values
+
+
+def _tiles(new, lengths, tq=16):
+    """What a step context hands the matrix-core kernel: tiles of up to ``tq`` tokens of one request."""
+    tile_req = [r for r, n in enumerate(new) for _ in range(-(-n // tq))]
+    tile_tok0 = [i * tq for n in new for i in range(-(-n // tq))]
+    indptr = [0]
+    for n in new:
+        indptr.append(indptr[-1] + n)
+    as_int = lambda v: torch.tensor(v, dtype=torch.int32).cuda()
+    return as_int(indptr), as_int([L - n for L, n in zip(lengths, new)]), as_int(tile_req), as_int(tile_tok0), len(tile_req)
 
 
 def _attend(q, keys, values, p, H, G, scale, cap, chunk, window):
@@ -126,27 +137,29 @@ def test_attention_with_cap_chunks_and_window(dtype, H, G, dim, vdim, page, chun
     for r, (L, n) in enumerate(zip(lengths, new)):
         for j in range(L - n):
             kd[table[r, j // page], :, j % page] = keys[r][j].cuda()
-            vd[table[r, j // page], :, j % page] = values[r][j].cuda()
+            vd[table[r, j // page], :, :, j % page] = values[r][j].cuda()
     k_new = torch.cat([keys[r][L - n:].reshape(n, -1) for r, (L, n) in enumerate(zip(lengths, new))])
     v_new = torch.cat([values[r][L - n:].reshape(n, -1) for r, (L, n) in enumerate(zip(lengths, new))])
     wide = torch.cat((k_new, v_new), dim=1).cuda()                  # row-strided views, as a mixer hands them over
     ops.kv_cache_write(wide[:, : G * dim], wide[:, G * dim:], token_req.cuda(), positions.cuda(), tab, kd, vd, page)
     for r, L in enumerate(lengths):
         j = L - 1
-        assert torch.equal(kd[table[r, j // page], :, j % page].cpu(), keys[r][j]) and torch.equal(vd[table[r, j // page], :, j % page].cpu(), values[r][j])
+        assert torch.equal(kd[table[r, j // page], :, j % page].cpu(), keys[r][j]) and torch.equal(vd[table[r, j // page], :, :, j % page].cpu(), values[r][j])
     assert bool(torch.isnan(kd[0].float()).all())                   # the sentinel page stays unwritten
     qs = torch.cat([x.reshape(x.shape[0], -1) for x in q]).cuda()
     out = torch.full((qs.shape[0], H * vdim + 5), float("nan"), dtype=dtype, device="cuda")
-    ops.local_attention(qs, out[:, 3: 3 + H * vdim], kd, vd, tab, token_req.cuda(), positions.cuda(), H, G, dim, vdim, page, scale, cap, chunk, window, gain,
-                        max_new_tokens=max(new))
+    ops.local_attention(qs, out[:, 3: 3 + H * vdim], kd, vd, tab, token_req.cuda(), positions.cuda(), H, G, dim, vdim, page, scale, cap, chunk, window, gain)
     want = torch.stack([gain * _attend(q[r][i], keys[r], values[r], lengths[r] - new[r] + i, H, G, scale, cap, chunk, window)
                         for r in range(3) for i in range(new[r])])
     torch.testing.assert_close(out[:, 3: 3 + H * vdim].cpu().double(), want, **_tol(dtype, 2))
     assert bool(torch.isnan(out[:, :3].float()).all() and torch.isnan(out[:, 3 + H * vdim:].float()).all())
-    if dtype == torch.bfloat16:                                     # the kernel without matrix cores on the same operands
-        general = torch.empty((qs.shape[0], H * vdim), dtype=dtype, device="cuda")
-        ops.local_attention(qs, general, kd, vd, tab, token_req.cuda(), positions.cuda(), H, G, dim, vdim, page, scale, cap, chunk, window, gain, general=True)
-        torch.testing.assert_close(general.cpu().double(), want, **_tol(dtype, 2))
+    assert ops.local_attention_mfma_fits(dtype, dim, vdim, page) == (dtype == torch.bfloat16 and dim in (64, 128) and page == 16)
+    if ops.local_attention_mfma_fits(dtype, dim, vdim, page):       # the matrix-core kernel on the same operands, in tiles of 16 tokens
+        tiled = torch.full((qs.shape[0], H * vdim + 8), float("nan"), dtype=dtype, device="cuda")
+        ops.local_attention(qs, tiled[:, 8:], kd, vd, tab, token_req.cuda(), positions.cuda(), H, G, dim, vdim, page, scale, cap, chunk, window, gain,
+                            tiles=_tiles(new, lengths))
+        torch.testing.assert_close(tiled[:, 8:].cpu().double(), want, **_tol(dtype, 2))
+        assert bool(torch.isnan(tiled[:, :8].float()).all())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -155,7 +168,7 @@ def test_one_key_at_the_edge_of_a_chunk_carries_the_weight(dtype, new):
     """The first key of the query's chunk is scaled up so that it takes nearly all the weight, and its value is unlike the others: the
     output shows whether it was read.  The key just before the chunk is scaled up as much in another run: it must not show."""
     from torchlet_amd.kernels import ops
-    H, G, dim, vdim, page, chunk = 2, 1, 32, 48, 16, 96
+    H, G, dim, vdim, page, chunk = 2, 1, 32, 64, 16, 96
     L = 96 * 3 + 57
     for edge, seen in ((96 * 3, True), (96 * 3 - 1, False)):
         g = torch.Generator().manual_seed(4)
@@ -166,15 +179,18 @@ def test_one_key_at_the_edge_of_a_chunk_carries_the_weight(dtype, new):
         kd, vd = k_plane.cuda(), v_plane.cuda()
         for j in range(L):
             kd[table[0, j // page], :, j % page] = keys[0][j].cuda()
-            vd[table[0, j // page], :, j % page] = values[0][j].cuda()
-        out = torch.empty((new, H * vdim), dtype=dtype, device="cuda")
+            vd[table[0, j // page], :, :, j % page] = values[0][j].cuda()
+        # pages before the query's chunk may have gone back to the pool: their table entries point at the sentinel page, which holds NaN here
+        tab = table.clone()
+        tab[0, : (96 * 3 - 1) // page] = 0
         token_req = torch.zeros(new, dtype=torch.int32).cuda()
         positions = torch.arange(L - new, L, dtype=torch.int32).cuda()
-        ops.local_attention(q.reshape(new, -1).cuda(), out, kd, vd, table.cuda(), token_req, positions, H, G, dim, vdim, page, 1.0, 0.0, chunk, 0, 1.0,
-                            max_new_tokens=new)
         want = _attend(q[-1], keys[0], values[0], L - 1, H, G, 1.0, 0.0, chunk, 0)
-        torch.testing.assert_close(out[-1].cpu().double(), want, **_tol(dtype, 50))
-        assert (float(out[-1, :vdim].float().mean()) > 90.0) == seen
+        for tiles in (None, _tiles([new], [L])) if dtype == torch.bfloat16 and new > 1 else (None,):
+            out = torch.empty((new, H * vdim), dtype=dtype, device="cuda")
+            ops.local_attention(q.reshape(new, -1).cuda(), out, kd, vd, tab.cuda(), token_req, positions, H, G, dim, vdim, page, 1.0, 0.0, chunk, 0, 1.0, tiles=tiles)
+            torch.testing.assert_close(out[-1].cpu().double(), want, **_tol(dtype, 50))
+            assert (float(out[-1, :vdim].float().mean()) > 90.0) == seen
 
 
 # ------------------------------------------------------------------ the gated delta rule
@@ -254,7 +270,7 @@ def test_delta_rule_against_plain_and_portions_to_the_bit(H, G, dim, vdim):
         return torch.cat((q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)), dim=1).contiguous(), gates.contiguous()
 
     (x1, g1), (x2, g2) = inputs(T1), inputs(T2)
-    extra = 5
+    extra = 8 if dim % 8 == 0 else 5            # rows of the state that are, and are not, aligned for 16-byte pieces
     start = torch.randn(3, H * dim * vdim + extra, generator=g) * 0.3
 
     def want(x, gates, S0):
@@ -262,14 +278,14 @@ def test_delta_rule_against_plain_and_portions_to_the_bit(H, G, dim, vdim):
         of = torch.arange(H) // (H // G)
         q, k = x[:, : G * dim].view(T, G, dim)[:, of].double(), x[:, G * dim: 2 * G * dim].view(T, G, dim)[:, of].double()
         v = x[:, 2 * G * dim:].view(T, H, vdim).double()
-        S = S0.double().view(H, dim, vdim).clone()
+        S = S0.double().view(H, vdim, dim).transpose(1, 2).clone()          # a head's state lies column by column
         out = []
         for t in range(T):
             S = S * gates[t, H:, None, None].double()
             u = gates[t, :H, None].double() * (v[t] - torch.einsum("hde,hd->he", S, k[t]))
             S = S + k[t][:, :, None] * u[:, None, :]
             out.append(torch.einsum("hde,hd->he", S, q[t]).reshape(-1))
-        return torch.stack(out), S.reshape(-1)
+        return torch.stack(out), S.transpose(1, 2).reshape(-1)
 
     def run(portions, slot_of):
         """``portions``: a list of steps, each a list of (request, tokens of it).  Returns the outputs per request and the state tensor."""

@@ -1,8 +1,9 @@
 // Attention over a paged cache whose keys and values differ in size (dim and vdim numbers per head), with soft-capped scores and a
 // local mask: a query at position p reads the keys j <= p of its own chunk (j / chunk == p / chunk, chunks counted from position 0)
 // and, with a window, j > p - window.  Scores, softmax and the weighted sum are float whatever the activation type.
-//   k_plane [pages, kv_heads, page_size, dim], v_plane [pages, kv_heads, page_size, vdim]; key j of a request lies in slot
-//   j % page_size of page block_table[request][j / page_size].
+//   k_plane [pages, kv_heads, page_size, dim], v_plane [pages, kv_heads, vdim, page_size] (the values of a page lie transposed, so
+//   that eight neighbouring keys' values of one column are 16 bytes side by side, which is how the matrix cores want them); key j
+//   of a request lies in slot j % page_size of page block_table[request][j / page_size].
 #include "common.h"
 
 // ------------------------------------------------------------------ cache write
@@ -23,7 +24,7 @@ __global__ void kv_cache_write_kernel(const T* __restrict__ k, int k_ld, const T
     }
     for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
         const int g = i / vdim, d = i % vdim;
-        v_plane[(((size_t)page * kv_heads + g) * page_size + slot) * vdim + d] = v[(size_t)t * v_ld + i];
+        v_plane[(((size_t)page * kv_heads + g) * vdim + d) * page_size + slot] = v[(size_t)t * v_ld + i];
     }
 }
 
@@ -95,11 +96,13 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
         const int j = lo + b * TL_WAVE + lane;
         const bool ok = j <= p;
         float s = -INFINITY;
-        size_t at = 0;                                 // the key's row in its plane, in rows of one head
+        size_t at = 0;                                 // page and head of the key, and its slot
+        int slot = 0;
         if (ok) {
             const int page = table[j / page_size];
-            at = ((size_t)page * kv_heads + g) * page_size + j % page_size;
-            const T* kr = k_plane + at * dim;
+            at = (size_t)page * kv_heads + g;
+            slot = j % page_size;
+            const T* kr = k_plane + (at * page_size + slot) * dim;
             float dot = 0.f;
             for (int d = 0; d < dim; ++d) dot = fmaf(sq[d], to_float(kr[d]), dot);
             s = cap_score(dot, cap);
@@ -114,12 +117,12 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
         const int nb = min(TL_WAVE, p - (lo + b * TL_WAVE) + 1);
         for (int i = 0; i < nb; ++i) {
             const float wi = __shfl(w, i, TL_WAVE);
-            const size_t ati = __shfl((unsigned long long)at, i, TL_WAVE);
-            const T* vr = v_plane + ati * vdim;
+            const size_t ati = ((size_t)(unsigned)__shfl((int)(at >> 32), i, TL_WAVE) << 32) | (unsigned)__shfl((int)at, i, TL_WAVE);
+            const T* vr = v_plane + ati * vdim * page_size + __shfl(slot, i, TL_WAVE);
 #pragma unroll
             for (int c = 0; c < LA_COLS; ++c) {
                 const int col = lane + c * TL_WAVE;
-                if (col < vdim) acc[c] = fmaf(wi, to_float(vr[col]), acc[c]);
+                if (col < vdim) acc[c] = fmaf(wi, to_float(vr[(size_t)col * page_size]), acc[c]);
             }
         }
     }
@@ -144,10 +147,222 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
     }
 }
 
+
+// ------------------------------------------------------------------ the matrix-core kernel (bfloat16, prompts)
+// One wave per tile of 16 consecutive tokens of a request and query head; the four waves of a work-group take four neighbouring
+// heads, which mostly share their keys and values.  Nothing passes through shared memory: with v_mfma_f32_16x16x32_bf16 the first
+// operand's lane holds 8 neighbouring k of one row, which for keys (rows of K, k along dim), queries (rows of Q, k along dim) and
+// transposed values (rows of V^T, k along the keys of a page) are 16 bytes side by side in memory.
+//   scores, transposed: S^T[key][token] = K Q^T.  A lane ends up with one token (lane % 16) and four keys (rows 4 q .. 4 q + 3, q = lane / 16)
+//   per product.  A step takes 32 keys in two products whose rows are keys base + 8 (r / 4) + r % 4 and that plus 4, so a lane holds
+//   the keys base + 8 q .. 8 q + 7 of its token: exactly the 8 neighbouring k of the second operand of
+//   O^T[column][token] += V^T[column][key] P^T[key][token], with no exchange between lanes.
+// Cap, mask, running maximum and sum are per token, that is per lane, with the maximum and the final sum joined across the four
+// lanes of a token.  Weights are rounded to bfloat16 for the second product; sums are float.
+typedef __bf16 la_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float la_f32x4 __attribute__((ext_vector_type(4)));
+union LaFrag {
+    uint4 u;
+    la_bf16x8 v;
+    uint16_t e[8];
+};
+#define LAM_TOKENS 16
+#define LAM_KEYS 32
+
+__device__ __forceinline__ float cap_score_fast(float s, float cap, float inv_cap) {
+    if (cap <= 0.f) return s;
+    // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2 x) + 1); beyond |x| = 15 it is +-1 to the last bit
+    const float x = fminf(fmaxf(s * inv_cap, -15.f), 15.f);
+    return cap * (1.f - 2.f / (expf(2.f * x) + 1.f));
+}
+
+template <int DK, int DV>          // dim / 32 and vdim / 16
+__global__ void __launch_bounds__(256)
+local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __restrict__ out, int out_ld, const bf16_t* __restrict__ k_plane,
+                            const bf16_t* __restrict__ v_plane, const int* __restrict__ block_table, int table_ld, int table_width,
+                            const int* __restrict__ req_indptr, const int* __restrict__ ctx_lens, const int* __restrict__ tile_req,
+                            const int* __restrict__ tile_tok0, int heads, int kv_heads, int page_size, float scale, float cap,
+                            LocalMask mask, float gain) {
+    constexpr int dim = DK * 32, vdim = DV * 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, kq = lane >> 4;
+    const int head = blockIdx.y * 4 + wave;
+    if (head >= heads) return;
+    const int tile = blockIdx.x;
+    const int req = tile_req ? tile_req[tile] : tile;
+    const int first = req_indptr[req], n_new = req_indptr[req + 1] - first;
+    const int tok0 = tile_tok0 ? tile_tok0[tile] : 0;
+    const int n_tile = min(LAM_TOKENS, n_new - tok0);            // tokens of this tile
+    if (n_tile <= 0) return;
+    const int g = head / (heads / kv_heads);
+    const int p0 = ctx_lens[req] + tok0;                         // position of the tile's first token
+    const int my_tok = min(li, n_tile - 1);                      // (lanes beyond the tile's tokens repeat its last one and store nothing)
+    const int my_p = p0 + my_tok, my_lo = mask.first(my_p);
+    const int* table = block_table + (size_t)req * table_ld;
+    const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+
+    LaFrag qf[DK];
+    {
+        const bf16_t* qrow = q + (size_t)(first + tok0 + my_tok) * q_ld + head * dim + 8 * kq;
+#pragma unroll
+        for (int s = 0; s < DK; ++s) qf[s].u = *(const uint4*)(qrow + 32 * s);
+    }
+    la_f32x4 acc[DV];
+#pragma unroll
+    for (int j = 0; j < DV; ++j) acc[j] = la_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    const int p_last = p0 + n_tile - 1;
+    const int lo_tile = mask.first(p0);                          // the first token reads furthest back; pages before may be gone
+    const int base0 = lo_tile / LAM_KEYS * LAM_KEYS;
+    // rows of the two score products that this lane fetches: keys base + 8 (li / 4) + li % 4 (+ 4)
+    const int krow = 8 * (li >> 2) + (li & 3);
+    // the keys of a step are fetched one step ahead: a step's own fetches are its values and the keys of the next one
+    LaFrag a0[DK], a1[DK];
+    auto fetch_keys = [&](int base) {
+        const int key0 = max(min(base + krow, p_last), lo_tile), key1 = max(min(base + krow + 4, p_last), lo_tile);       // (clamped: masked below)
+        const bf16_t* k0 = k_plane + (((size_t)table[key0 / page_size] * kv_heads + g) * page_size + key0 % page_size) * dim + 8 * kq;
+        const bf16_t* k1 = k_plane + (((size_t)table[key1 / page_size] * kv_heads + g) * page_size + key1 % page_size) * dim + 8 * kq;
+#pragma unroll
+        for (int s = 0; s < DK; ++s) { a0[s].u = *(const uint4*)(k0 + 32 * s); a1[s].u = *(const uint4*)(k1 + 32 * s); }
+    };
+    fetch_keys(base0);
+    for (int base = base0; base <= p_last; base += LAM_KEYS) {
+        // ---- scores of 32 keys
+        la_f32x4 s0 = la_f32x4{0.f, 0.f, 0.f, 0.f}, s1 = la_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DK; ++s) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[s].v, qf[s].v, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[s].v, qf[s].v, s1, 0, 0, 0);
+        }
+        if (base + LAM_KEYS <= p_last) fetch_keys(base + LAM_KEYS);
+        // ---- the values of these keys, transposed: row = column of the values, k = keys base + 8 kq .. + 7 (one page: page_size % 8 == 0)
+        LaFrag vf[DV];
+        {
+            const int key = base + 8 * kq;
+            const int kc = max(min(key, p_last), lo_tile);
+            const bf16_t* vt = v_plane + (((size_t)table[kc / page_size] * kv_heads + g) * vdim + li) * page_size + key % page_size;
+#pragma unroll
+            for (int j = 0; j < DV; ++j) {
+                vf[j].u = (key <= p_last && key + 7 >= lo_tile) ? *(const uint4*)(vt + (size_t)16 * j * page_size) : uint4{0u, 0u, 0u, 0u};
+                if (key + 7 > p_last || key < lo_tile) {        // places no token has written yet, or whose page is gone, may hold anything
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (key + e > p_last || key + e < lo_tile) vf[j].e[e] = 0;
+                }
+            }
+        }
+        // ---- cap, mask, running maximum
+        float sc[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int key = base + 8 * kq + e;
+            const float raw = (e < 4 ? s0[e] : s1[e - 4]) * scale;
+            sc[e] = (key <= my_p && key >= my_lo) ? cap_score_fast(raw, cap, inv_cap) : -INFINITY;
+            mx = fmaxf(mx, sc[e]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, TL_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, TL_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a token that has seen no key yet
+        const float keep = expf(m - m_use);                     // (0 while m is -inf)
+        m = m_new;
+        LaFrag pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float w = expf(sc[e] - m_use);
+            const bf16_t wb = from_float<bf16_t>(w);
+            pf.e[e] = wb.bits;
+            psum += to_float(wb);                               // the sum of what the second product sees
+        }
+        l = l * keep + psum;
+#pragma unroll
+        for (int j = 0; j < DV; ++j) {
+            acc[j][0] *= keep; acc[j][1] *= keep; acc[j][2] *= keep; acc[j][3] *= keep;
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j].v, pf.v, acc[j], 0, 0, 0);
+        }
+    }
+    l += __shfl_xor(l, 16, TL_WAVE);
+    l += __shfl_xor(l, 32, TL_WAVE);
+    if (li >= n_tile) return;
+    const float norm = gain / l;
+    // acc[j][v] = O[token li][column 16 j + 4 kq + v]
+    bf16_t* orow = out + (size_t)(first + tok0 + li) * out_ld + head * vdim + 4 * kq;
+#pragma unroll
+    for (int j = 0; j < DV; ++j) {
+        union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[j][v] * norm).bits;
+        if ((out_ld & 3) == 0 && ((uintptr_t)out & 7) == 0) *(uint2*)(orow + 16 * j) = pk.u;
+        else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) orow[16 * j + v].bits = pk.e[v];
+        }
+    }
+}
+
+template <int DK, int DV>
+static void launch_local_mfma(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, const void* block_table,
+                              int table_ld, int table_width, const void* req_indptr, const void* ctx_lens, const void* tile_req,
+                              const void* tile_tok0, int tiles, int heads, int kv_heads, int page_size, float scale, float cap, LocalMask mask,
+                              float gain, hipStream_t stream) {
+    dim3 grid(tiles, (heads + 3) / 4), block(256);
+    local_attention_mfma_kernel<DK, DV><<<grid, block, 0, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, out_ld, (const bf16_t*)k_plane, (const bf16_t*)v_plane,
+        (const int*)block_table, table_ld, table_width, (const int*)req_indptr, (const int*)ctx_lens, (const int*)tile_req, (const int*)tile_tok0,
+        heads, kv_heads, page_size, scale, cap, mask, gain);
+}
+
+// Whether the matrix-core kernel is built for these sizes.
+extern "C" int tl_local_attention_mfma_fits(int dim, int vdim, int page_size) {
+    const bool dk = dim == 32 || dim == 64 || dim == 96 || dim == 128 || dim == 192 || dim == 256;
+    const bool dv = vdim == 16 || vdim == 32 || vdim == 64 || vdim == 96 || vdim == 128 || vdim == 192 || vdim == 256;
+    return dk && dv && page_size % 8 == 0;
+}
+
+// Tiles of up to 16 consecutive tokens of one request: tile i belongs to request tile_req[i] (null: request i) and starts at that
+// request's token tile_tok0[i] of the step (null: 0).
+extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, int pages,
+                                        const void* block_table, int table_ld, int table_width, const void* req_indptr, const void* ctx_lens,
+                                        const void* tile_req, const void* tile_tok0, int tiles, int heads, int kv_heads, int dim, int vdim,
+                                        int page_size, float scale, float cap, int chunk, int window, float gain, hipStream_t stream) {
+    TL_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && page_size > 0, "local_attention_tiles: bad sizes");
+    TL_REQUIRE(tl_local_attention_mfma_fits(dim, vdim, page_size), "local_attention_tiles: not built for heads of %d / %d numbers in pages of %d", dim, vdim, page_size);
+    TL_REQUIRE(q_ld >= heads * dim && q_ld % 8 == 0 && ((uintptr_t)q & 15) == 0 && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0,
+               "local_attention_tiles: rows too short or not aligned");
+    if (tiles == 0) return TL_OK;
+    const LocalMask mask{chunk, window};
+#define TL_LAM(DK, DV)                                                                                                                      \
+    launch_local_mfma<DK, DV>(q, q_ld, out, out_ld, k_plane, v_plane, block_table, table_ld, table_width, req_indptr, ctx_lens, tile_req,  \
+                              tile_tok0, tiles, heads, kv_heads, page_size, scale, cap, mask, gain, stream)
+#define TL_LAM_V(DK)                                     \
+    switch (vdim) {                                      \
+        case 16: TL_LAM(DK, 1); break;                   \
+        case 32: TL_LAM(DK, 2); break;                   \
+        case 64: TL_LAM(DK, 4); break;                   \
+        case 96: TL_LAM(DK, 6); break;                   \
+        case 128: TL_LAM(DK, 8); break;                  \
+        case 192: TL_LAM(DK, 12); break;                 \
+        default: TL_LAM(DK, 16); break;                  \
+    }
+    switch (dim) {
+        case 32: TL_LAM_V(1) break;
+        case 64: TL_LAM_V(2) break;
+        case 96: TL_LAM_V(3) break;
+        case 128: TL_LAM_V(4) break;
+        case 192: TL_LAM_V(6) break;
+        default: TL_LAM_V(8) break;
+    }
+#undef TL_LAM_V
+#undef TL_LAM
+    TL_CHECK_LAUNCH("local_attention_mfma");
+    return TL_OK;
+}
+
 extern "C" int tl_local_attention(const void* q, int q_ld, void* out, int out_ld, const void* k_plane, const void* v_plane, int pages,
                                   const void* block_table, int table_ld, int table_width, const void* token_req, const void* positions,
                                   int tokens, int heads, int kv_heads, int dim, int vdim, int page_size, float scale, float cap, int chunk,
-                                  int window, float gain, int longest, int general, int dtype, hipStream_t stream) {
+                                  int window, float gain, int dtype, hipStream_t stream) {
     TL_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0, "local_attention: bad sizes");
     TL_REQUIRE(dim <= LA_MAX_DIM && vdim <= LA_MAX_DIM, "local_attention: built for heads of up to %d numbers, got %d / %d", LA_MAX_DIM, dim, vdim);
     TL_REQUIRE(q_ld >= heads * dim && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0, "local_attention: rows too short");

@@ -466,47 +466,70 @@ extern "C" int tl_delta_prepare(const void* proj, int ld, const void* conv_w, vo
 //   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q.
 // Column j of S needs only its own a_j = sum_r S[r][j] k[r] and b_j = sum_r S[r][j] q[r] (of the state before the decay) and k . q:
 //   u_j = beta (v_j - g a_j);   o_j = g b_j + (k . q) u_j;   S[r][j] <- g S[r][j] + k[r] u_j.
-// A lane owns DELTA_RPL rows of one column in registers for all tokens of the step; L = 1 .. 16 lanes (a power of two, fixed by dim
-// alone) share a column and add their sums by exchanging across the wave, always in the same order, so a token's result depends
-// neither on how its request was cut into steps nor on what else the step holds.  A wave has 64 / L columns, a work-group of four
-// waves four times that: neighbouring columns, so that the rows of the state are fetched in whole lines.  Tokens are taken TB at a
-// time: their q, k, v, beta and g go to shared memory (the next batch is fetched into registers while this one is worked on), every
-// lane runs the TB updates of its rows, and the outputs leave through shared memory.
-#define DELTA_RPL 16
+// The 16 lanes of a row of the wave share a column: lane i of them owns the rows i RPL .. i RPL + RPL - 1 of it in registers for all
+// tokens of the step (RPL = 4, 8, 12 or 16, fixed by dim alone), and they add their sums with four exchanges inside the row (pairs,
+// quads, halves, the row: every lane gets the same bits).  The order of every sum is fixed by dim, so a token's result depends neither
+// on how its request was cut into steps nor on what else the step holds.  A wave has 4 columns, a work-group of four waves 16.  The
+// state of a head lies column by column ([vdim][dim]), so a lane's rows are side by side in memory and a wave fetches whole lines.
+// Tokens are taken TB at a time: their q, k, v, beta and g go to shared memory (the next batch is fetched into registers while this one
+// is worked on) and every lane runs the TB updates of its rows.
+#define DELTA_L 16
+#define DELTA_COLS 16           // columns of a work-group
 #define DELTA_TB 16
 
+template <int CTRL>
+__device__ __forceinline__ float row_exchange(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// The sum of v over the 16 lanes of a row of the wave, in every one of them.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += row_exchange<0xB1>(v);        // quad_perm [1, 0, 3, 2]: the neighbour
+    v += row_exchange<0x4E>(v);        // quad_perm [2, 3, 0, 1]: the other pair of the quad
+    v += row_exchange<0x141>(v);       // row_half_mirror: the other quad of the half
+    v += row_exchange<0x140>(v);       // row_mirror: the other half
+    return v;
+}
+
+template <int RPL>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, float* __restrict__ state, size_t slot_stride,
                   const int* __restrict__ slots, const int* __restrict__ req_indptr, float* __restrict__ out,
-                  int heads, int kv_heads, int dim, int vdim, int L, int tb) {
+                  int heads, int kv_heads, int dim, int vdim, int tb) {
     extern __shared__ float smem[];
-    const int CW = TL_WAVE / L;                        // columns of a wave
-    const int cols = 4 * CW;                           // ... of the work-group
-    const int rows_pad = L * DELTA_RPL;                // >= dim
-    float* sq = smem;                                  // [tb][rows_pad]
-    float* sk = sq + tb * rows_pad;                    // [tb][rows_pad]
-    float* sv = sk + tb * rows_pad;                    // [tb][cols]
-    float* sg = sv + tb * cols;                        // [tb][2]: beta, decay
-    float* so = sg + tb * 2;                           // [tb][cols]
-    const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * cols;
+    constexpr int ROWS = DELTA_L * RPL;                // >= dim
+    float* sq = smem;                                  // [tb][ROWS]
+    float* sk = sq + tb * ROWS;                        // [tb][ROWS]
+    float* sv = sk + tb * ROWS;                        // [tb][DELTA_COLS]
+    float* sg = sv + tb * DELTA_COLS;                  // [tb][2]: beta, decay
+    const int req = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * DELTA_COLS;
     const int tok0 = req_indptr[req], tok1 = req_indptr[req + 1];
     if (tok0 >= tok1) return;
     const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
-    const int rg = lane / CW, cw = lane % CW;          // the lane's group of rows and its column within the wave
-    const int col = col0 + wave * CW + cw, row0 = rg * DELTA_RPL;
+    const int rg = lane & 15, cw = wave * 4 + (lane >> 4);       // the lane's group of rows and its column within the work-group
+    const int col = col0 + cw, row0 = rg * RPL;
     const bool col_ok = col < vdim;
     const int C = 2 * kv_heads * dim + heads * vdim;
     const int qk_head = head / (heads / kv_heads);
     const int q_at = qk_head * dim, k_at = kv_heads * dim + qk_head * dim, v_at = 2 * kv_heads * dim + head * vdim + col0;
-    float* st = state + (size_t)slots[req] * slot_stride + (size_t)head * dim * vdim;
+    float* st = state + (size_t)slots[req] * slot_stride + ((size_t)head * vdim + col) * dim + row0;
 
-    float S[DELTA_RPL];
+    float S[RPL];
+    const bool whole = col_ok && row0 + RPL <= dim && (dim & 3) == 0 && ((uintptr_t)state & 15) == 0 && (slot_stride & 3) == 0;
+    if (whole) {
 #pragma unroll
-    for (int r = 0; r < DELTA_RPL; ++r) S[r] = (col_ok && row0 + r < dim) ? st[(size_t)(row0 + r) * vdim + col] : 0.f;
+        for (int r = 0; r < RPL; r += 4) {
+            const float4 x = *(const float4*)(st + r);
+            S[r] = x.x; S[r + 1] = x.y; S[r + 2] = x.z; S[r + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) S[r] = (col_ok && row0 + r < dim) ? st[r] : 0.f;
+    }
 
-    // a batch's numbers, fetched into registers one batch ahead: per token 2 * rows_pad of q and k (zeros beyond dim), cols of v, 2 gates
-    const int per_token = 2 * rows_pad + cols + 2;
-    constexpr int STAGE = (DELTA_TB * (2 * 16 * DELTA_RPL + 4 * TL_WAVE + 2) + 255) / 256;       // at most, per thread
+    // a batch's numbers, fetched into registers one batch ahead: per token 2 * ROWS of q and k (zeros beyond dim), 16 of v, 2 gates
+    constexpr int PER_TOKEN = 2 * ROWS + DELTA_COLS + 2;
+    constexpr int STAGE = (DELTA_TB * PER_TOKEN + 255) / 256;
     float stage[STAGE];
     auto fetch = [&](int base) {
         const int nb = min(tb, tok1 - base);
@@ -514,13 +537,13 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
         for (int j = 0; j < STAGE; ++j) {
             const int idx = threadIdx.x + j * 256;
             float v = 0.f;
-            if (idx < nb * per_token) {
-                const int t = idx / per_token, e = idx % per_token;
+            if (idx < nb * PER_TOKEN) {
+                const int t = idx / PER_TOKEN, e = idx % PER_TOKEN;
                 const float* row = qkv + (size_t)(base + t) * C;
-                if (e < rows_pad) v = e < dim ? row[q_at + e] : 0.f;
-                else if (e < 2 * rows_pad) v = e - rows_pad < dim ? row[k_at + e - rows_pad] : 0.f;
-                else if (e < 2 * rows_pad + cols) v = col0 + e - 2 * rows_pad < vdim ? row[v_at + e - 2 * rows_pad] : 0.f;
-                else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * rows_pad - cols) * heads + head];
+                if (e < ROWS) v = e < dim ? row[q_at + e] : 0.f;
+                else if (e < 2 * ROWS) v = e - ROWS < dim ? row[k_at + e - ROWS] : 0.f;
+                else if (e < 2 * ROWS + DELTA_COLS) v = col0 + e - 2 * ROWS < vdim ? row[v_at + e - 2 * ROWS] : 0.f;
+                else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
             }
             stage[j] = v;
         }
@@ -528,77 +551,80 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
     fetch(tok0);
     for (int base = tok0; base < tok1; base += tb) {
         const int nb = min(tb, tok1 - base);
-        __syncthreads();                               // the batch before has been worked on and its outputs have left
+        __syncthreads();                               // the batch before has been worked on
 #pragma unroll
         for (int j = 0; j < STAGE; ++j) {
             const int idx = threadIdx.x + j * 256;
-            if (idx < nb * per_token) {
-                const int t = idx / per_token, e = idx % per_token;
-                if (e < rows_pad) sq[t * rows_pad + e] = stage[j];
-                else if (e < 2 * rows_pad) sk[t * rows_pad + e - rows_pad] = stage[j];
-                else if (e < 2 * rows_pad + cols) sv[t * cols + e - 2 * rows_pad] = stage[j];
-                else sg[t * 2 + e - 2 * rows_pad - cols] = stage[j];
+            if (idx < nb * PER_TOKEN) {
+                const int t = idx / PER_TOKEN, e = idx % PER_TOKEN;
+                if (e < ROWS) sq[t * ROWS + e] = stage[j];
+                else if (e < 2 * ROWS) sk[t * ROWS + e - ROWS] = stage[j];
+                else if (e < 2 * ROWS + DELTA_COLS) sv[t * DELTA_COLS + e - 2 * ROWS] = stage[j];
+                else sg[t * 2 + e - 2 * ROWS - DELTA_COLS] = stage[j];
             }
         }
         if (base + tb < tok1) fetch(base + tb);
         __syncthreads();
+        float* orow = out + ((size_t)base * heads + head) * vdim + col;
+#pragma unroll 2
         for (int t = 0; t < nb; ++t) {
-            const float* kt = sk + t * rows_pad + row0;
-            const float* qt = sq + t * rows_pad + row0;
-            float kr[DELTA_RPL], qr[DELTA_RPL];
+            const float* kt = sk + t * ROWS + row0;
+            const float* qt = sq + t * ROWS + row0;
+            float kr[RPL], qr[RPL];
 #pragma unroll
-            for (int r = 0; r < DELTA_RPL; r += 4) {
+            for (int r = 0; r < RPL; r += 4) {
                 const float4 k4 = *(const float4*)(kt + r), q4 = *(const float4*)(qt + r);
                 kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
                 qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
             }
+            const float beta = sg[t * 2], g = sg[t * 2 + 1], vt = sv[t * DELTA_COLS + cw];
             // four chains of additions each, joined in a fixed order
             float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int r = 0; r < DELTA_RPL; ++r) {
+            for (int r = 0; r < RPL; ++r) {
                 a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
                 b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
                 c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
             }
-            float a = (a4[0] + a4[1]) + (a4[2] + a4[3]), b = (b4[0] + b4[1]) + (b4[2] + b4[3]), kq = (c4[0] + c4[1]) + (c4[2] + c4[3]);
-            for (int o = CW; o < TL_WAVE; o <<= 1) {   // the other groups of rows of this column
-                a += __shfl_xor(a, o, TL_WAVE);
-                b += __shfl_xor(b, o, TL_WAVE);
-                kq += __shfl_xor(kq, o, TL_WAVE);
-            }
-            const float beta = sg[t * 2], g = sg[t * 2 + 1];
-            const float u = beta * (sv[t * cols + wave * CW + cw] - g * a);
+            const float a = row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3]));
+            const float b = row16_sum((b4[0] + b4[1]) + (b4[2] + b4[3]));
+            const float kq = row16_sum((c4[0] + c4[1]) + (c4[2] + c4[3]));
+            const float u = beta * (vt - g * a);
 #pragma unroll
-            for (int r = 0; r < DELTA_RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
-            if (rg == 0) so[t * cols + wave * CW + cw] = fmaf(kq, u, g * b);
-        }
-        __syncthreads();
-        for (int idx = threadIdx.x; idx < nb * cols; idx += 256) {
-            const int t = idx / cols, c = idx % cols;
-            if (col0 + c < vdim) out[((size_t)(base + t) * heads + head) * vdim + col0 + c] = so[idx];
+            for (int r = 0; r < RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
+            if (rg == 0 && col_ok) orow[(size_t)t * heads * vdim] = fmaf(kq, u, g * b);
         }
     }
-    if (col_ok) {
+    if (whole) {
 #pragma unroll
-        for (int r = 0; r < DELTA_RPL; ++r)
-            if (row0 + r < dim) st[(size_t)(row0 + r) * vdim + col] = S[r];
+        for (int r = 0; r < RPL; r += 4) *(float4*)(st + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else if (col_ok) {
+#pragma unroll
+        for (int r = 0; r < RPL; ++r)
+            if (row0 + r < dim) st[r] = S[r];
     }
 }
 
+// state: per slot, from its start, heads x [vdim][dim] floats (a head's state column by column).
 extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, long slot_stride, const void* slots, const void* req_indptr,
                              void* out, int requests, int heads, int kv_heads, int dim, int vdim, int longest, hipStream_t stream) {
     TL_REQUIRE(requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0, "delta_scan: bad sizes");
-    TL_REQUIRE(dim <= 16 * DELTA_RPL, "delta_scan: built for up to %d query/key dimensions per head, got %d", 16 * DELTA_RPL, dim);
+    TL_REQUIRE(dim <= DELTA_L * 16, "delta_scan: built for up to %d query/key dimensions per head, got %d", DELTA_L * 16, dim);
     TL_REQUIRE(slot_stride >= (long)heads * dim * vdim, "delta_scan: the state rows are too short");
+    TL_REQUIRE(requests <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for one launch");
     if (requests == 0) return TL_OK;
-    int L = 1;
-    while (L * DELTA_RPL < dim) L *= 2;
-    const int cols = 4 * (TL_WAVE / L);
+    const int rpl = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 192 ? 12 : 16;
     const int tb = longest < 1 ? 1 : (longest < DELTA_TB ? longest : DELTA_TB);
-    const size_t smem = sizeof(float) * (size_t)tb * (2 * L * DELTA_RPL + 2 * cols + 2);
-    dim3 grid((vdim + cols - 1) / cols, heads, requests), block(256);
-    delta_scan_kernel<<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride, (const int*)slots,
-                                                     (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim, L, tb);
+    const size_t smem = sizeof(float) * (size_t)tb * (2 * DELTA_L * rpl + DELTA_COLS + 2);
+    dim3 grid((vdim + DELTA_COLS - 1) / DELTA_COLS, heads, requests), block(256);
+#define TL_DELTA(R)                                                                                                                        \
+    delta_scan_kernel<R><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride,       \
+                                                        (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim, tb)
+    if (rpl == 4) TL_DELTA(4);
+    else if (rpl == 8) TL_DELTA(8);
+    else if (rpl == 12) TL_DELTA(12);
+    else TL_DELTA(16);
+#undef TL_DELTA
     TL_CHECK_LAUNCH("delta_scan");
     return TL_OK;
 }

@@ -901,7 +901,7 @@ def delta_scan(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, slot
                heads: int, kv_heads: int, dim: int, vdim: int, max_new_tokens: int | None = None) -> None:
     """The gated delta rule over the step's tokens, request by request from the state its slot holds: ``qkv`` float32 ``[T, C]`` as
     :func:`delta_prepare` left it (queries, keys, values), ``gates`` float32 ``[T, 2 * heads]`` (beta, decay); head ``h`` of ``state[slot]``
-    (float32, ``dim x vdim`` numbers from ``h * dim * vdim`` on) moves by ``S <- g S; u = beta (v - S^T k); S <- S + k u^T`` and ``out`` float32
+    (float32, ``dim x vdim`` numbers from ``h * dim * vdim`` on, column by column: ``[vdim][dim]``) moves by ``S <- g S; u = beta (v - S^T k); S <- S + k u^T`` and ``out`` float32
     ``[T, heads * vdim]`` receives ``S^T q``."""
     T = qkv.shape[0]
     R = req_indptr.numel() - 1
@@ -929,17 +929,19 @@ LOCAL_ATTENTION_MAX_DIM = 256
 
 def _check_local_planes(what, k_plane, v_plane, dtype, kv_heads, dim, vdim, page_size):
     if k_plane.dtype != dtype or v_plane.dtype != dtype or not k_plane.is_contiguous() or not v_plane.is_contiguous() \
-            or k_plane.shape[1:] != (kv_heads, page_size, dim) or v_plane.shape[1:] != (kv_heads, page_size, vdim) or k_plane.shape[0] != v_plane.shape[0]:
-        raise KernelError(f"{what}: cache planes {tuple(k_plane.shape)} / {tuple(v_plane.shape)} are not [pages, {kv_heads}, {page_size}, {dim} / {vdim}] of {dtype}")
+            or k_plane.shape[1:] != (kv_heads, page_size, dim) or v_plane.shape[1:] != (kv_heads, vdim, page_size) or k_plane.shape[0] != v_plane.shape[0]:
+        raise KernelError(f"{what}: cache planes {tuple(k_plane.shape)} / {tuple(v_plane.shape)} are not [pages, {kv_heads}, {page_size}, {dim}] and "
+                          f"[pages, {kv_heads}, {vdim}, {page_size}] of {dtype}")
 
 
 def kv_cache_write(k: torch.Tensor, v: torch.Tensor, token_req: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    k_plane: torch.Tensor, v_plane: torch.Tensor, page_size: int) -> None:
     """The step's keys ``k [T, kv_heads * dim]`` and values ``v [T, kv_heads * vdim]`` (row-strided views) go to their places in the pages:
     token ``t`` of request ``token_req[t]`` at position ``p`` to slot ``p % page_size`` of page ``block_table[request, p // page_size]`` of
-    ``k_plane [pages, kv_heads, page_size, dim]`` and ``v_plane [pages, kv_heads, page_size, vdim]``.  What would go to page 0 is dropped."""
+    ``k_plane [pages, kv_heads, page_size, dim]`` and ``v_plane [pages, kv_heads, vdim, page_size]`` (the values of a page lie transposed).
+    What would go to page 0 is dropped."""
     T = k.shape[0]
-    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[3]
+    kv_heads, dim, vdim = k_plane.shape[1], k_plane.shape[3], v_plane.shape[2]
     _check_local_planes("kv_cache_write", k_plane, v_plane, k.dtype, kv_heads, dim, vdim, page_size)
     if k.shape != (T, kv_heads * dim) or v.shape != (T, kv_heads * vdim) or k.stride(1) != 1 or v.stride(1) != 1 or v.dtype != k.dtype:
         raise KernelError("kv_cache_write: keys or values do not fit the planes")
@@ -953,32 +955,56 @@ def kv_cache_write(k: torch.Tensor, v: torch.Tensor, token_req: torch.Tensor, po
                                       _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]), c_int(page_size), c_int(_dt(k, "kv_cache_write")), _stream()))
 
 
+LOCAL_ATTENTION_TILE_TOKENS = 16      # tokens of a tile of the matrix-core kernel
+
+
+def local_attention_mfma_fits(dtype: torch.dtype, dim: int, vdim: int, page_size: int) -> bool:
+    """Whether the matrix-core kernel of :func:`local_attention` is built for these sizes (bfloat16; key sizes 32, 64, 96, 128, 192, 256;
+    value sizes 16, 32, 64, 96, 128, 192, 256; pages of a multiple of 8 tokens)."""
+    return dtype == torch.bfloat16 and bool(_lib("local_attention").tl_local_attention_mfma_fits(c_int(dim), c_int(vdim), c_int(page_size)))
+
+
 def local_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor, block_table: torch.Tensor,
                     token_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, page_size: int,
-                    scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0,
-                    max_new_tokens: int | None = None, general: bool = False) -> None:
+                    scale: float, softcap: float = 0.0, chunk: int = 0, window: int = 0, gain: float = 1.0, tiles=None) -> None:
     """Attention of the step's queries ``q [T, heads * dim]`` over their requests' cached keys and values (which hold the step's own tokens
     already): query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then (``softcap > 0``) ``softcap *
     tanh(score / softcap)``; a query at position ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (``chunk > 0``) and ``j > p -
     window`` (``window > 0``); softmax and weighted sum in 32-bit; ``out [T, heads * vdim]`` receives the result times ``gain``.  ``q`` and ``out``
-    may be row-strided views.  ``max_new_tokens``: the most tokens a request brings in this step, if known (steps of single tokens skip
-    the kernel that tiles prompts); ``general=True`` forces the kernel without matrix cores."""
+    may be row-strided views.  Without ``tiles`` one work-group per token and head walks the keys (every dtype and size).  ``tiles =
+    (req_indptr, ctx_lens, tile_req, tile_tok0, number of tiles)`` (tiles of up to 16 consecutive tokens of one request, as a step
+    context makes them) runs the matrix-core kernel, where :func:`local_attention_mfma_fits` says it is built."""
     T = q.shape[0]
     _check_local_planes("local_attention", k_plane, v_plane, q.dtype, kv_heads, dim, vdim, page_size)
     if q.shape != (T, heads * dim) or out.shape != (T, heads * vdim) or q.stride(1) != 1 or out.stride(1) != 1 or out.dtype != q.dtype \
             or heads % kv_heads or max(dim, vdim) > LOCAL_ATTENTION_MAX_DIM:
         raise KernelError("local_attention: queries or output do not fit")
-    _i32(token_req, "token_req", T)
-    _i32(positions, "positions", T)
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
         raise KernelError("local_attention: the block table must be int32 [requests, blocks]")
     lib = _lib("local_attention")
+    if tiles is not None:
+        req_indptr, ctx_lens, tile_req, tile_tok0, n_tiles = tiles
+        if not local_attention_mfma_fits(q.dtype, dim, vdim, page_size) or q.stride(0) % 8 or q.data_ptr() % 16:
+            raise KernelError("local_attention: the matrix-core kernel is not built for these operands")
+        R = block_table.shape[0]
+        _i32(req_indptr, "req_indptr", R + 1)
+        _i32(ctx_lens, "ctx_lens", R)
+        _i32(tile_req, "tile_req", n_tiles)
+        _i32(tile_tok0, "tile_tok0", n_tiles)
+        if tile_req is None and n_tiles > R:
+            raise KernelError("local_attention: without a tile list there is one tile per request")
+        _check(lib, lib.tl_local_attention_tiles(_ptr(q), c_int(q.stride(0)), _ptr(out), c_int(out.stride(0)), _ptr(k_plane), _ptr(v_plane),
+                                                 c_int(k_plane.shape[0]), _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]),
+                                                 _ptr(req_indptr), _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(n_tiles), c_int(heads),
+                                                 c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale), c_float(softcap),
+                                                 c_int(chunk), c_int(window), c_float(gain), _stream()))
+        return
+    _i32(token_req, "token_req", T)
+    _i32(positions, "positions", T)
     _check(lib, lib.tl_local_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), c_int(out.stride(0)), _ptr(k_plane), _ptr(v_plane), c_int(k_plane.shape[0]),
                                        _ptr(block_table), c_int(block_table.stride(0)), c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions),
                                        c_int(T), c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(page_size), c_float(scale),
-                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain),
-                                       c_int(T if max_new_tokens is None else max_new_tokens), c_int(1 if general else 0),
-                                       c_int(_dt(q, "local_attention")), _stream()))
+                                       c_float(softcap), c_int(chunk), c_int(window), c_float(gain), c_int(_dt(q, "local_attention")), _stream()))
 
 
 # ------------------------------------------------------------- attention over a cached latent

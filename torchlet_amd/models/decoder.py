@@ -73,7 +73,7 @@ class DecoderModel:
         return plan
 
     def tile_token_sizes(self) -> set[int]:
-        return {b.mixer.tile_tokens for b in self.blocks if hasattr(b.mixer, "tile_tokens")}
+        return {p.tile_tokens for p in self.parts() if hasattr(p, "tile_tokens")}
 
     def parts(self):
         """Every part of the model: each block with what is inside it, and the final norm."""

@@ -4,8 +4,11 @@
 encoding; query head ``i`` reads key/value head ``i // (heads / kv_heads)``; ``score = q . k * scale``, then ``score <- cap *
 tanh(score / cap)``; query ``p`` reads the keys ``j <= p`` with ``j // chunk == p // chunk`` (chunks are counted from position 0 of
 the sequence, whatever portion a step brings) and, with a window, ``j > p - window``; an ordinary softmax in 32-bit; ``W_o`` on the
-heads' values side by side.  The cache has two planes per page, ``[kv_heads, page, dim]`` and ``[kv_heads, page, vdim]``; pages that
-lie wholly before the chunk of a request's next position go back to the pool.
+heads' values side by side.  The cache has two planes per page, keys ``[kv_heads, page, dim]`` and values, transposed, ``[kv_heads, vdim,
+page]``; pages that lie wholly before the chunk of a request's next position go back to the pool.  The bfloat16 engine runs on the matrix
+cores in tiles of up to 16 tokens of a request, a wave to a tile and head (where the kernel is built for the sizes: a decoded token is
+a tile of one, and the fetches of its keys are what its time is made of either way); the 32-bit engine and other sizes take the kernel
+that walks the keys of one token and head.
 """
 from __future__ import annotations
 
@@ -36,6 +39,7 @@ class CappedAttention(StagedMixer):
         self.scale = float(spec.scale)
         self.softcap = float(spec.softcap) if spec.softcap else 0.0
         self.chunk, self.window = spec.chunk or 0, spec.window or 0
+        self.tile_tokens = ops.LOCAL_ATTENTION_TILE_TOKENS       # the step context makes tiles of this many tokens ahead of the layers
 
     def paged_need(self):
         return PagedNeed(num_heads=self.kv_heads, head_dim=self.dim, window=self.spec.window, chunk=self.spec.chunk,
@@ -53,11 +57,17 @@ class CappedAttention(StagedMixer):
         self.w_o = self._place(tensors["o"], KEEP_COMPUTE)
 
     def mix(self, proj, h, ctx, cache, out, gain=1.0):
+        # the cache hands out planes of [pages, kv_heads, page, width]; this mixer keeps the values of a page transposed
         k_plane, v_plane = cache.planes
+        v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.vdim, cache.page_size)
         table = ctx.block_tables[cache.group]
         q = proj[:, : self.q_width]
         if cache.writable:
             ops.kv_cache_write(proj[:, self.q_width: self.q_width + self.k_width], proj[:, self.q_width + self.k_width:],
                                ctx.token_req, ctx.positions, table, k_plane, v_plane, cache.page_size)
+        tiles = None
+        if h.is_cuda and ops.local_attention_mfma_fits(self.dtype, self.dim, self.vdim, cache.page_size) \
+                and proj.stride(0) % 8 == 0 and proj.data_ptr() % 16 == 0:
+            tiles = (ctx.req_indptr, ctx.ctx_lens, *ctx.tiles(ops.LOCAL_ATTENTION_TILE_TOKENS))
         ops.local_attention(q, out, k_plane, v_plane, table, ctx.token_req, ctx.positions, self.heads, self.kv_heads, self.dim, self.vdim,
-                            cache.page_size, self.scale, self.softcap, self.chunk, self.window, gain, max_new_tokens=ctx.max_new_tokens)
+                            cache.page_size, self.scale, self.softcap, self.chunk, self.window, gain, tiles=tiles)
