@@ -149,8 +149,10 @@ local_attention_kernel(const T* __restrict__ q, int q_ld, T* __restrict__ out, i
 
 
 // ------------------------------------------------------------------ the matrix-core kernel (bfloat16, prompts)
-// One wave per tile of 16 consecutive tokens of a request and query head; the four waves of a work-group take four neighbouring
-// heads, which mostly share their keys and values.  Nothing passes through shared memory: with v_mfma_f32_16x16x32_bf16 the first
+// One work-group of four waves per tile of 16 consecutive tokens of a request and query head.  The tile's keys come in steps of 32, dealt
+// to the waves in turn (step i to wave i % 4: a matter of the positions alone), so that the longest tile of a step, whose time is the
+// chain of its steps, takes a quarter of them per wave; the four waves' running maxima, sums and outputs are joined through shared
+// memory at the end.  The operands do not pass through shared memory: with v_mfma_f32_16x16x32_bf16 the first
 // operand's lane holds 8 neighbouring k of one row, which for keys (rows of K, k along dim), queries (rows of Q, k along dim) and
 // transposed values (rows of V^T, k along the keys of a page) are 16 bytes side by side in memory.
 //   scores, transposed: S^T[key][token] = K Q^T.  A lane ends up with one token (lane % 16) and four keys (rows 4 q .. 4 q + 3, q = lane / 16)
@@ -168,12 +170,17 @@ union LaFrag {
 };
 #define LAM_TOKENS 16
 #define LAM_KEYS 32
+#define LAM_WAVES 4
+#define LAM_STRIDE (LAM_WAVES * LAM_KEYS)      // keys from one step of a wave to its next
 
-__device__ __forceinline__ float cap_score_fast(float s, float cap, float inv_cap) {
+// The hardware's own 2^x and 1 / x (about one unit in the last place each): a tile's time is these, eight scores to a lane and step.
+#define LA_LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ float cap_score_fast(float s, float cap, float two_log2e_over_cap) {
     if (cap <= 0.f) return s;
-    // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2 x) + 1); beyond |x| = 15 it is +-1 to the last bit
-    const float x = fminf(fmaxf(s * inv_cap, -15.f), 15.f);
-    return cap * (1.f - 2.f / (expf(2.f * x) + 1.f));
+    // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (e^(2 x) + 1); beyond |x| = 15 it is +-1 to the last bit
+    const float e = __builtin_amdgcn_exp2f(fminf(fmaxf(s * two_log2e_over_cap, -43.f), 43.f));
+    return cap * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
 }
 
 template <int DK, int DV>          // dim / 32 and vdim / 16
@@ -184,9 +191,9 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
                             const int* __restrict__ tile_tok0, int heads, int kv_heads, int page_size, float scale, float cap,
                             LocalMask mask, float gain) {
     constexpr int dim = DK * 32, vdim = DV * 16;
+    extern __shared__ float la_smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, kq = lane >> 4;
-    const int head = blockIdx.y * 4 + wave;
-    if (head >= heads) return;
+    const int head = blockIdx.y;
     const int tile = blockIdx.x;
     const int req = tile_req ? tile_req[tile] : tile;
     const int first = req_indptr[req], n_new = req_indptr[req + 1] - first;
@@ -198,7 +205,11 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
     const int my_tok = min(li, n_tile - 1);                      // (lanes beyond the tile's tokens repeat its last one and store nothing)
     const int my_p = p0 + my_tok, my_lo = mask.first(my_p);
     const int* table = block_table + (size_t)req * table_ld;
-    const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+    const float inv_cap = cap > 0.f ? 2.f * LA_LOG2E / cap : 0.f;
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    const int page_shift = __ffs(page_size) - 1;
+    auto page_of = [&](int key) { return pow2 ? key >> page_shift : key / page_size; };
+    auto slot_of = [&](int key) { return pow2 ? key & (page_size - 1) : key % page_size; };
 
     LaFrag qf[DK];
     {
@@ -216,17 +227,32 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
     const int base0 = lo_tile / LAM_KEYS * LAM_KEYS;
     // rows of the two score products that this lane fetches: keys base + 8 (li / 4) + li % 4 (+ 4)
     const int krow = 8 * (li >> 2) + (li & 3);
-    // the keys of a step are fetched one step ahead: a step's own fetches are its values and the keys of the next one
-    LaFrag a0[DK], a1[DK];
-    auto fetch_keys = [&](int base) {
-        const int key0 = max(min(base + krow, p_last), lo_tile), key1 = max(min(base + krow + 4, p_last), lo_tile);       // (clamped: masked below)
-        const bf16_t* k0 = k_plane + (((size_t)table[key0 / page_size] * kv_heads + g) * page_size + key0 % page_size) * dim + 8 * kq;
-        const bf16_t* k1 = k_plane + (((size_t)table[key1 / page_size] * kv_heads + g) * page_size + key1 % page_size) * dim + 8 * kq;
+    // The pages of up to 64 blocks of the request lie in a register across the wave (lane i: block tab_first + i) and are read from
+    // there, so that no fetch waits for a look-up in memory; the window moves on every 64 blocks.
+    int tab_first = page_of(base0);
+    int tab_reg = table[min(tab_first + lane, table_width - 1)];
+    auto page_at = [&](int key) { return __shfl(tab_reg, page_of(key) - tab_first, TL_WAVE); };
+    // The keys and values of a step are fetched one step ahead, while the step before is worked on.
+    LaFrag a0[DK], a1[DK], va[DV], vb[DV];
+    auto fetch = [&](int base, LaFrag (&vf)[DV]) {
+        if (page_of(base + LAM_KEYS - 1) - tab_first >= TL_WAVE) {            // (the same for every lane)
+            tab_first = page_of(base);
+            tab_reg = table[min(tab_first + lane, table_width - 1)];
+        }
+        // keys: rows base + krow and base + krow + 4 (clamped into what exists: masked below)
+        const int key0 = max(min(base + krow, p_last), lo_tile), key1 = max(min(base + krow + 4, p_last), lo_tile);
+        const bf16_t* k0 = k_plane + (((size_t)page_at(key0) * kv_heads + g) * page_size + slot_of(key0)) * dim + 8 * kq;
+        const bf16_t* k1 = k_plane + (((size_t)page_at(key1) * kv_heads + g) * page_size + slot_of(key1)) * dim + 8 * kq;
 #pragma unroll
         for (int s = 0; s < DK; ++s) { a0[s].u = *(const uint4*)(k0 + 32 * s); a1[s].u = *(const uint4*)(k1 + 32 * s); }
+        // values, transposed: row = column of the values, k = keys base + 8 kq .. + 7 (one page: page_size % 8 == 0)
+        const int key = base + 8 * kq;
+        const int kc = max(min(key, p_last), lo_tile);
+        const bf16_t* vt = v_plane + (((size_t)page_at(kc) * kv_heads + g) * vdim + li) * page_size + slot_of(key);
+#pragma unroll
+        for (int j = 0; j < DV; ++j) vf[j].u = *(const uint4*)(vt + (size_t)16 * j * page_size);      // (never conditional: nothing waits for it here)
     };
-    fetch_keys(base0);
-    for (int base = base0; base <= p_last; base += LAM_KEYS) {
+    auto step = [&](int base, LaFrag (&vf)[DV], LaFrag (&vnext)[DV]) {
         // ---- scores of 32 keys
         la_f32x4 s0 = la_f32x4{0.f, 0.f, 0.f, 0.f}, s1 = la_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -234,71 +260,81 @@ local_attention_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, bf16_t* __re
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[s].v, qf[s].v, s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[s].v, qf[s].v, s1, 0, 0, 0);
         }
-        if (base + LAM_KEYS <= p_last) fetch_keys(base + LAM_KEYS);
-        // ---- the values of these keys, transposed: row = column of the values, k = keys base + 8 kq .. + 7 (one page: page_size % 8 == 0)
-        LaFrag vf[DV];
-        {
-            const int key = base + 8 * kq;
-            const int kc = max(min(key, p_last), lo_tile);
-            const bf16_t* vt = v_plane + (((size_t)table[kc / page_size] * kv_heads + g) * vdim + li) * page_size + key % page_size;
-#pragma unroll
-            for (int j = 0; j < DV; ++j) {
-                vf[j].u = (key <= p_last && key + 7 >= lo_tile) ? *(const uint4*)(vt + (size_t)16 * j * page_size) : uint4{0u, 0u, 0u, 0u};
-                if (key + 7 > p_last || key < lo_tile) {        // places no token has written yet, or whose page is gone, may hold anything
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (key + e > p_last || key + e < lo_tile) vf[j].e[e] = 0;
-                }
-            }
-        }
-        // ---- cap, mask, running maximum
+        if (base + LAM_STRIDE <= p_last) fetch(base + LAM_STRIDE, vnext);
+        // ---- cap, mask, running maximum (scores in units of log 2 from here on, so that the weights are plain powers of two)
         float sc[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int key = base + 8 * kq + e;
             const float raw = (e < 4 ? s0[e] : s1[e - 4]) * scale;
-            sc[e] = (key <= my_p && key >= my_lo) ? cap_score_fast(raw, cap, inv_cap) : -INFINITY;
+            sc[e] = (key <= my_p && key >= my_lo) ? cap_score_fast(raw, cap, inv_cap) * LA_LOG2E : -INFINITY;
             mx = fmaxf(mx, sc[e]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, TL_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, TL_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a token that has seen no key yet
-        const float keep = expf(m - m_use);                     // (0 while m is -inf)
+        const float keep = __builtin_amdgcn_exp2f(m - m_use);   // (0 while m is -inf)
         m = m_new;
         LaFrag pf;
         float psum = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float w = expf(sc[e] - m_use);
+            const float w = __builtin_amdgcn_exp2f(sc[e] - m_use);
             const bf16_t wb = from_float<bf16_t>(w);
             pf.e[e] = wb.bits;
             psum += to_float(wb);                               // the sum of what the second product sees
         }
         l = l * keep + psum;
+        // places no token has written yet, or whose page is gone, may hold anything: their values count as zero (first and last steps only)
+        const int vkey = base + 8 * kq;
+        if (vkey + 7 > p_last || vkey < lo_tile) {
 #pragma unroll
-        for (int j = 0; j < DV; ++j) {
-            acc[j][0] *= keep; acc[j][1] *= keep; acc[j][2] *= keep; acc[j][3] *= keep;
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j].v, pf.v, acc[j], 0, 0, 0);
+            for (int j = 0; j < DV; ++j)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (vkey + e > p_last || vkey + e < lo_tile) vf[j].e[e] = 0;
+        }
+        if (__any(keep != 1.f)) {                               // (the maxima settle after a tile's first steps)
+#pragma unroll
+            for (int j = 0; j < DV; ++j) { acc[j][0] *= keep; acc[j][1] *= keep; acc[j][2] *= keep; acc[j][3] *= keep; }
+        }
+#pragma unroll
+        for (int j = 0; j < DV; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j].v, pf.v, acc[j], 0, 0, 0);
+    };
+    if (base0 + LAM_KEYS * wave <= p_last) {
+        fetch(base0 + LAM_KEYS * wave, va);
+        for (int base = base0 + LAM_KEYS * wave; base <= p_last; base += 2 * LAM_STRIDE) {
+            step(base, va, vb);
+            if (base + LAM_STRIDE <= p_last) step(base + LAM_STRIDE, vb, va);
         }
     }
     l += __shfl_xor(l, 16, TL_WAVE);
     l += __shfl_xor(l, 32, TL_WAVE);
-    if (li >= n_tile) return;
-    const float norm = gain / l;
+    // ---- the four waves' shares are joined: per token the maxima, the sums and the outputs, in the order of the waves
+    float* sm_m = la_smem;                              // [4][16], in units of log 2
+    float* sm_l = sm_m + LAM_WAVES * LAM_TOKENS;        // [4][16]
+    float* sm_o = sm_l + LAM_WAVES * LAM_TOKENS;        // [4][16][vdim]
+    if (kq == 0) { sm_m[wave * LAM_TOKENS + li] = m; sm_l[wave * LAM_TOKENS + li] = l; }
     // acc[j][v] = O[token li][column 16 j + 4 kq + v]
-    bf16_t* orow = out + (size_t)(first + tok0 + li) * out_ld + head * vdim + 4 * kq;
 #pragma unroll
-    for (int j = 0; j < DV; ++j) {
-        union { uint2 u; uint16_t e[4]; } pk;
+    for (int j = 0; j < DV; ++j)
+        *(float4*)(sm_o + ((size_t)wave * LAM_TOKENS + li) * vdim + 16 * j + 4 * kq) = make_float4(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < n_tile * vdim; idx += blockDim.x) {
+        const int tok = idx / vdim, col = idx % vdim;
+        float top = sm_m[tok];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[j][v] * norm).bits;
-        if ((out_ld & 3) == 0 && ((uintptr_t)out & 7) == 0) *(uint2*)(orow + 16 * j) = pk.u;
-        else {
+        for (int w = 1; w < LAM_WAVES; ++w) top = fmaxf(top, sm_m[w * LAM_TOKENS + tok]);
+        float den = 0.f, o = 0.f;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) orow[16 * j + v].bits = pk.e[v];
+        for (int w = 0; w < LAM_WAVES; ++w) {
+            const float f = __builtin_amdgcn_exp2f(sm_m[w * LAM_TOKENS + tok] - top);        // (0 for a wave that saw no key of this token)
+            den = fmaf(sm_l[w * LAM_TOKENS + tok], f, den);
+            o = fmaf(sm_o[((size_t)w * LAM_TOKENS + tok) * vdim + col], f, o);
         }
+        out[(size_t)(first + tok0 + tok) * out_ld + head * vdim + col] = from_float<bf16_t>(o * (gain / den));
     }
 }
 
@@ -307,8 +343,15 @@ static void launch_local_mfma(const void* q, int q_ld, void* out, int out_ld, co
                               int table_ld, int table_width, const void* req_indptr, const void* ctx_lens, const void* tile_req,
                               const void* tile_tok0, int tiles, int heads, int kv_heads, int page_size, float scale, float cap, LocalMask mask,
                               float gain, hipStream_t stream) {
-    dim3 grid(tiles, (heads + 3) / 4), block(256);
-    local_attention_mfma_kernel<DK, DV><<<grid, block, 0, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, out_ld, (const bf16_t*)k_plane, (const bf16_t*)v_plane,
+    dim3 grid(tiles, heads), block(LAM_WAVES * TL_WAVE);
+    const size_t smem = sizeof(float) * LAM_WAVES * LAM_TOKENS * (2 + DV * 16);
+    auto kernel = local_attention_mfma_kernel<DK, DV>;
+    static bool raised = false;                      // (per instance of the template)
+    if (smem > 48 * 1024 && !raised) {
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        raised = true;
+    }
+    kernel<<<grid, block, smem, stream>>>((const bf16_t*)q, q_ld, (bf16_t*)out, out_ld, (const bf16_t*)k_plane, (const bf16_t*)v_plane,
         (const int*)block_table, table_ld, table_width, (const int*)req_indptr, (const int*)ctx_lens, (const int*)tile_req, (const int*)tile_tok0,
         heads, kv_heads, page_size, scale, cap, mask, gain);
 }
@@ -326,7 +369,7 @@ extern "C" int tl_local_attention_tiles(const void* q, int q_ld, void* out, int 
                                         const void* block_table, int table_ld, int table_width, const void* req_indptr, const void* ctx_lens,
                                         const void* tile_req, const void* tile_tok0, int tiles, int heads, int kv_heads, int dim, int vdim,
                                         int page_size, float scale, float cap, int chunk, int window, float gain, hipStream_t stream) {
-    TL_REQUIRE(tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && page_size > 0, "local_attention_tiles: bad sizes");
+    TL_REQUIRE(tiles >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && heads % kv_heads == 0 && page_size > 0, "local_attention_tiles: bad sizes");
     TL_REQUIRE(tl_local_attention_mfma_fits(dim, vdim, page_size), "local_attention_tiles: not built for heads of %d / %d numbers in pages of %d", dim, vdim, page_size);
     TL_REQUIRE(q_ld >= heads * dim && q_ld % 8 == 0 && ((uintptr_t)q & 15) == 0 && out_ld >= heads * vdim && table_ld >= table_width && chunk >= 0 && window >= 0,
                "local_attention_tiles: rows too short or not aligned");

@@ -565,34 +565,45 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
         }
         if (base + tb < tok1) fetch(base + tb);
         __syncthreads();
-        float* orow = out + ((size_t)base * heads + head) * vdim + col;
-#pragma unroll 2
-        for (int t = 0; t < nb; ++t) {
-            const float* kt = sk + t * ROWS + row0;
-            const float* qt = sq + t * ROWS + row0;
-            float kr[RPL], qr[RPL];
+        // the batch's tokens one after the other, the loop written out: nothing in it writes memory, so the fetches of the tokens to
+        // come move ahead of the sums of the token at hand; the outputs wait in registers for the end of the batch
+        float obuf[DELTA_TB];
 #pragma unroll
-            for (int r = 0; r < RPL; r += 4) {
-                const float4 k4 = *(const float4*)(kt + r), q4 = *(const float4*)(qt + r);
-                kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
-                qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+        for (int t = 0; t < DELTA_TB; ++t) {
+            obuf[t] = 0.f;
+            if (t < nb) {
+                const float* kt = sk + t * ROWS + row0;
+                const float* qt = sq + t * ROWS + row0;
+                float kr[RPL], qr[RPL];
+#pragma unroll
+                for (int r = 0; r < RPL; r += 4) {
+                    const float4 k4 = *(const float4*)(kt + r), q4 = *(const float4*)(qt + r);
+                    kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
+                    qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+                }
+                const float beta = sg[t * 2], g = sg[t * 2 + 1], vt = sv[t * DELTA_COLS + cw];
+                // four chains of additions each, joined in a fixed order
+                float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < RPL; ++r) {
+                    a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
+                    b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
+                    c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
+                }
+                const float a = row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3]));
+                const float b = row16_sum((b4[0] + b4[1]) + (b4[2] + b4[3]));
+                const float kq = row16_sum((c4[0] + c4[1]) + (c4[2] + c4[3]));
+                const float u = beta * (vt - g * a);
+#pragma unroll
+                for (int r = 0; r < RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
+                obuf[t] = fmaf(kq, u, g * b);
             }
-            const float beta = sg[t * 2], g = sg[t * 2 + 1], vt = sv[t * DELTA_COLS + cw];
-            // four chains of additions each, joined in a fixed order
-            float a4[4] = {0.f, 0.f, 0.f, 0.f}, b4[4] = {0.f, 0.f, 0.f, 0.f}, c4[4] = {0.f, 0.f, 0.f, 0.f};
+        }
+        if (rg == 0 && col_ok) {
+            float* orow = out + ((size_t)base * heads + head) * vdim + col;
 #pragma unroll
-            for (int r = 0; r < RPL; ++r) {
-                a4[r & 3] = fmaf(S[r], kr[r], a4[r & 3]);
-                b4[r & 3] = fmaf(S[r], qr[r], b4[r & 3]);
-                c4[r & 3] = fmaf(kr[r], qr[r], c4[r & 3]);
-            }
-            const float a = row16_sum((a4[0] + a4[1]) + (a4[2] + a4[3]));
-            const float b = row16_sum((b4[0] + b4[1]) + (b4[2] + b4[3]));
-            const float kq = row16_sum((c4[0] + c4[1]) + (c4[2] + c4[3]));
-            const float u = beta * (vt - g * a);
-#pragma unroll
-            for (int r = 0; r < RPL; ++r) S[r] = fmaf(kr[r], u, g * S[r]);
-            if (rg == 0 && col_ok) orow[(size_t)t * heads * vdim] = fmaf(kq, u, g * b);
+            for (int t = 0; t < DELTA_TB; ++t)
+                if (t < nb) orow[(size_t)t * heads * vdim] = obuf[t];
         }
     }
     if (whole) {
