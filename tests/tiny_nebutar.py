@@ -52,8 +52,8 @@ CONFIGS = {
     ]),
     # every token takes the one expert: nothing hangs on a choice; far-away context reaches the logits through the recurrent state
     "S": dict(architecture="Nebutar", vocab=80, width=64, max_positions=512, norm=dict(eps=1e-5), embedding=dict(scale=3.0), streams=2, layers=[
-        _layer(_left(4, 1, 16, 32, 0.25, softcap=20.0, chunk=32), _right(2, 2, 16, 24, 3), 0.8, 1.0, _moe(48, 1, 0, 1)),
-        _layer(_left(4, 2, 16, 32, 0.25, softcap=20.0, chunk=48), _right(4, 1, 32, 16, 3), 0.8, 1.0, _moe(48, 1, 0, 1)),
+        _layer(_left(4, 1, 16, 32, 0.25, softcap=15.0, chunk=32), _right(2, 2, 16, 24, 3), 0.8, 1.0, _moe(48, 1, 0, 1)),
+        _layer(_left(4, 2, 16, 32, 0.25, softcap=25.0, chunk=48), _right(4, 1, 32, 16, 3), 0.8, 1.0, _moe(48, 1, 0, 1)),
     ]),
 }
 SEEDS = {"A": 13, "B": 14, "C": 16, "S": 18}
