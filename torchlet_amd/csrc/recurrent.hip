@@ -471,8 +471,9 @@ extern "C" int tl_delta_prepare(const void* proj, int ld, const void* conv_w, vo
 // quads, halves, the row: every lane gets the same bits).  The order of every sum is fixed by dim, so a token's result depends neither
 // on how its request was cut into steps nor on what else the step holds.  A wave has 4 columns, a work-group of four waves 16.  The
 // state of a head lies column by column ([vdim][dim]), so a lane's rows are side by side in memory and a wave fetches whole lines.
-// Tokens are taken TB at a time: their q, k, v, beta and g go to shared memory (the next batch is fetched into registers while this one
-// is worked on) and every lane runs the TB updates of its rows.
+// Tokens are taken TB at a time (1, 4 or 16, by the longest portion of the step): their q, k, v, beta and g go to shared memory (the
+// next batch is fetched into registers while this one is worked on) and every lane runs the TB updates of its rows; a request's last
+// batch is filled up with tokens that change nothing (k = 0, beta = 0, decay 1), so the loop has no branch.
 #define DELTA_L 16
 #define DELTA_COLS 16           // columns of a work-group
 #define DELTA_TB 16
@@ -491,11 +492,12 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-template <int RPL>
+template <int RPL, int TB>
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates, float* __restrict__ state, size_t slot_stride,
                   const int* __restrict__ slots, const int* __restrict__ req_indptr, float* __restrict__ out,
-                  int heads, int kv_heads, int dim, int vdim, int tb) {
+                  int heads, int kv_heads, int dim, int vdim) {
+    constexpr int tb = TB;
     extern __shared__ float smem[];
     constexpr int ROWS = DELTA_L * RPL;                // >= dim
     float* sq = smem;                                  // [tb][ROWS]
@@ -529,7 +531,7 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
 
     // a batch's numbers, fetched into registers one batch ahead: per token 2 * ROWS of q and k (zeros beyond dim), 16 of v, 2 gates
     constexpr int PER_TOKEN = 2 * ROWS + DELTA_COLS + 2;
-    constexpr int STAGE = (DELTA_TB * PER_TOKEN + 255) / 256;
+    constexpr int STAGE = (TB * PER_TOKEN + 255) / 256;
     float stage[STAGE];
     auto fetch = [&](int base) {
         const int nb = min(tb, tok1 - base);
@@ -537,13 +539,15 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
         for (int j = 0; j < STAGE; ++j) {
             const int idx = threadIdx.x + j * 256;
             float v = 0.f;
-            if (idx < nb * PER_TOKEN) {
+            if (idx < TB * PER_TOKEN) {
                 const int t = idx / PER_TOKEN, e = idx % PER_TOKEN;
-                const float* row = qkv + (size_t)(base + t) * C;
-                if (e < ROWS) v = e < dim ? row[q_at + e] : 0.f;
-                else if (e < 2 * ROWS) v = e - ROWS < dim ? row[k_at + e - ROWS] : 0.f;
-                else if (e < 2 * ROWS + DELTA_COLS) v = col0 + e - 2 * ROWS < vdim ? row[v_at + e - 2 * ROWS] : 0.f;
-                else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
+                if (t < nb) {
+                    const float* row = qkv + (size_t)(base + t) * C;
+                    if (e < ROWS) v = e < dim ? row[q_at + e] : 0.f;
+                    else if (e < 2 * ROWS) v = e - ROWS < dim ? row[k_at + e - ROWS] : 0.f;
+                    else if (e < 2 * ROWS + DELTA_COLS) v = col0 + e - 2 * ROWS < vdim ? row[v_at + e - 2 * ROWS] : 0.f;
+                    else v = gates[(size_t)(base + t) * 2 * heads + (e - 2 * ROWS - DELTA_COLS) * heads + head];
+                } else if (e == PER_TOKEN - 1) v = 1.f;        // beyond the request's last token: k = 0, beta = 0 and a decay of 1 leave the state as it is, to the bit
             }
             stage[j] = v;
         }
@@ -555,7 +559,7 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
 #pragma unroll
         for (int j = 0; j < STAGE; ++j) {
             const int idx = threadIdx.x + j * 256;
-            if (idx < nb * PER_TOKEN) {
+            if (idx < TB * PER_TOKEN) {
                 const int t = idx / PER_TOKEN, e = idx % PER_TOKEN;
                 if (e < ROWS) sq[t * ROWS + e] = stage[j];
                 else if (e < 2 * ROWS) sk[t * ROWS + e - ROWS] = stage[j];
@@ -565,13 +569,13 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
         }
         if (base + tb < tok1) fetch(base + tb);
         __syncthreads();
-        // the batch's tokens one after the other, the loop written out: nothing in it writes memory, so the fetches of the tokens to
-        // come move ahead of the sums of the token at hand; the outputs wait in registers for the end of the batch
-        float obuf[DELTA_TB];
+        // the batch's tokens one after the other, the loop written out without a branch (a batch is always whole: see above): nothing
+        // in it writes memory, so the fetches of the tokens to come move ahead of the sums of the token at hand; the outputs wait in
+        // registers for the end of the batch
+        float obuf[TB];
 #pragma unroll
-        for (int t = 0; t < DELTA_TB; ++t) {
-            obuf[t] = 0.f;
-            if (t < nb) {
+        for (int t = 0; t < TB; ++t) {
+            {
                 const float* kt = sk + t * ROWS + row0;
                 const float* qt = sq + t * ROWS + row0;
                 float kr[RPL], qr[RPL];
@@ -602,7 +606,7 @@ delta_scan_kernel(const float* __restrict__ qkv, const float* __restrict__ gates
         if (rg == 0 && col_ok) {
             float* orow = out + ((size_t)base * heads + head) * vdim + col;
 #pragma unroll
-            for (int t = 0; t < DELTA_TB; ++t)
+            for (int t = 0; t < TB; ++t)
                 if (t < nb) orow[(size_t)t * heads * vdim] = obuf[t];
         }
     }
@@ -625,17 +629,23 @@ extern "C" int tl_delta_scan(const void* qkv, const void* gates, void* state, lo
     TL_REQUIRE(requests <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for one launch");
     if (requests == 0) return TL_OK;
     const int rpl = dim <= 64 ? 4 : dim <= 128 ? 8 : dim <= 192 ? 12 : 16;
-    const int tb = longest < 1 ? 1 : (longest < DELTA_TB ? longest : DELTA_TB);
+    // tokens of a batch: 1 for a step of single tokens, 4 for short portions, else 16 (a batch is always worked through whole)
+    const int tb = longest <= 1 ? 1 : (longest <= 4 ? 4 : DELTA_TB);
     const size_t smem = sizeof(float) * (size_t)tb * (2 * DELTA_L * rpl + DELTA_COLS + 2);
     dim3 grid((vdim + DELTA_COLS - 1) / DELTA_COLS, heads, requests), block(256);
-#define TL_DELTA(R)                                                                                                                        \
-    delta_scan_kernel<R><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride,       \
-                                                        (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim, tb)
-    if (rpl == 4) TL_DELTA(4);
-    else if (rpl == 8) TL_DELTA(8);
-    else if (rpl == 12) TL_DELTA(12);
-    else TL_DELTA(16);
+#define TL_DELTA_B(R, B)                                                                                                                   \
+    delta_scan_kernel<R, B><<<grid, block, smem, stream>>>((const float*)qkv, (const float*)gates, (float*)state, (size_t)slot_stride,    \
+                                                           (const int*)slots, (const int*)req_indptr, (float*)out, heads, kv_heads, dim, vdim)
+#define TL_DELTA(R)                        \
+    if (tb == 1) TL_DELTA_B(R, 1);         \
+    else if (tb == 4) TL_DELTA_B(R, 4);    \
+    else TL_DELTA_B(R, DELTA_TB)
+    if (rpl == 4) { TL_DELTA(4); }
+    else if (rpl == 8) { TL_DELTA(8); }
+    else if (rpl == 12) { TL_DELTA(12); }
+    else { TL_DELTA(16); }
 #undef TL_DELTA
+#undef TL_DELTA_B
     TL_CHECK_LAUNCH("delta_scan");
     return TL_OK;
 }
